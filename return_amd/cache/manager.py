@@ -237,7 +237,7 @@ class CacheManager:
         full = -(-total_tokens // P)
         out = []
         for grp in self.groups:
-            w = grp.spec.window
+            w = None if grp.spec.keep_first else grp.spec.window
             if w is None:
                 out.append(full)
             else:
@@ -375,7 +375,7 @@ class CacheManager:
             if r is None:
                 continue
             for g, grp in enumerate(self.groups):
-                w = grp.spec.window
+                w = None if grp.spec.keep_first else grp.spec.window
                 if w is None:
                     continue
                 # the next query sits at position seq_len and reads keys >= seq_len - w + 1
@@ -418,7 +418,7 @@ class CacheManager:
                 assert r.first_pos[g] % P == 0
                 end = r.first_pos[g] + len(r.pages[g]) * P
                 assert r.seq_len <= end, f"{rid!r}: {r.seq_len} tokens but pages end at {end}"
-                if grp.spec.window is None:
+                if grp.spec.window is None or grp.spec.keep_first:
                     assert r.first_pos[g] == 0
                     assert len(r.pages[g]) == -(-r.seq_len // P), f"{rid!r}: page count off"
         slots = [r.slot for r in self.live.values()]

@@ -11,11 +11,14 @@ class PagedKVSpec:
 
     window None: every key stays until the request ends. window w: a query at
     position p reads keys at positions p-w+1..p, and pages that lie wholly before
-    that are given back while the request still runs.
+    that are given back while the request still runs. keep_first n: the keys at positions
+    below n stay readable whatever the window; the cache manager then keeps every page of the
+    request (the kernels skip what lies between the kept keys and the window).
     """
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    keep_first: int = 0
 
 
 @dataclasses.dataclass(frozen=True)

@@ -137,7 +137,7 @@ def load_config(path: str) -> ModelConfig:
         raise ConfigError(f"no config.json at {path}")
     with open(path) as f:
         raw = json.load(f)
-    arch = raw.get("architectures") or [None]
+    arch = raw.get("architectures") or [raw.get("architecture")]     # (a list, or one name under "architecture")
     if not arch[0]:
         raise ConfigError(f"{path}: no 'architectures' entry")
     cls, _ = lookup_architecture(arch[0])

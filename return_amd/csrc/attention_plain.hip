@@ -20,6 +20,11 @@
 // through LDS in wave order. Within a chunk four lanes share a key (each a quarter of the
 // head's elements, 16 bytes at a time), 16 keys at once; for the values the lanes run along the
 // head's elements, one key after the other.
+//
+// Optional, each off at 0 / null: head_scale[h] multiplies the scale of query head h; softcap c
+// turns a score s into c tanh(s / c); keep_first n lets every query also read the keys at positions
+// below n, whatever the window; sink adds one to the softmax's denominator (a key of score 0 that
+// has no value).
 #include "common.h"
 
 #define PLAIN_MAX_ACC 8     // D <= 64 * 8
@@ -43,7 +48,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
     const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ tok_ids, int n_seqs, int T_tokens, int Hq, int Hkv, int D, int P, float scale,
-    int window) {
+    int window, const float* __restrict__ head_scale, float softcap, int keep_first, int sink) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     float* q_s = smem;                                   // [QR][D]
     float* p_s = q_s + QR * D;                           // [WAVES][QR][64]
@@ -54,6 +59,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, part = lane & 3, sub = lane >> 2;
     const int head = blockIdx.y, kvh = head / (Hq / Hkv);
     const bool vec = (D & 3) == 0;
+    if (head_scale != nullptr) scale *= head_scale[head];
+    const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
 
     // the rows of this workgroup: token row, request, position; bit r of todo: row r is still to do
     int t_of[QR], seg_of[QR], pos_of[QR];
@@ -119,8 +126,13 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
 
         const int c_first = lo_pos / PLAIN_CHUNK;
         int c = c_first + ((wave - c_first) % WAVES + WAVES) % WAVES;      // first chunk >= c_first of this wave
+        // with kept first keys the pass begins at position 0 and leaves out the chunks that lie wholly
+        // between the kept keys and the first key of the rows' windows
+        const int low = (keep_first > 0 && lo_pos > 0) ? 0 : lo_pos;
+        if (low != lo_pos) c = wave;
         for (; c * PLAIN_CHUNK <= hi_pos; c += WAVES) {
             const int base = c * PLAIN_CHUNK;
+            if (base >= keep_first && base + PLAIN_CHUNK <= lo_pos) continue;
             // ---- scores: 16 keys at once, four lanes to a key
             float sc[4][QR];
 #pragma unroll
@@ -129,7 +141,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
                 const int p = base + kk;
                 const int idx = p - start;
                 const int pi = idx >= 0 ? idx / P : 0;
-                const bool there = p >= lo_pos && p <= hi_pos && pi < n_listed;   // else: not a key of this pass
+                const bool there = p >= low && (p >= lo_pos || p < keep_first) && p <= hi_pos && idx >= 0 &&
+                                   pi < n_listed;                                // else: not a key of this pass
                 const int row = there ? (pt[pi] * Hkv + kvh) * P + (idx - pi * P) : -1;   // [page][kv head][row in page]
                 float dot[QR];
 #pragma unroll
@@ -162,8 +175,10 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
                     float d = dot[r];
                     d += __shfl_xor(d, 1, 64);
                     d += __shfl_xor(d, 2, 64);
-                    const bool ok = there && active[r] && p <= pos_of[r] && p >= first_of[r];
-                    sc[sp][r] = ok ? d * scale : -INFINITY;
+                    const bool ok = there && active[r] && p <= pos_of[r] && (p >= first_of[r] || p < keep_first);
+                    d *= scale;
+                    if (softcap > 0.f) d = softcap * tanhf(d * inv_cap);
+                    sc[sp][r] = ok ? d : -INFINITY;
                 }
                 if (part == 0) my_row[kk] = row;
             }
@@ -241,6 +256,7 @@ __global__ __launch_bounds__(WAVES * 64) void attn_plain_kernel(
                 num = fmaf(acc_s[(w * QR + r) * D + e], ew, num);
                 den = fmaf(ml_s[(w * QR + r) * 2 + 1], ew, den);
             }
+            if (sink) den += expf(-mm);                  // one more key of score 0 that has no value
             out[((size_t)t_row * Hq + head) * D + e] = from_f<T>(den > 0.f ? num / den : 0.f);
         }
         __syncthreads();                                 // before the next pass writes q_s and the merge buffers
@@ -251,20 +267,22 @@ template <typename T, int QR, int WAVES>
 static void plain_launch(hipStream_t st, const void* q, void* out, const void* k_pool, const void* v_pool,
                          const int* page_table, const int* cu_pages, const int* kv_start, const int* cu_q,
                          const int* q_start, const int* tok_ids, int n_seqs, int T_tokens, int Hq, int Hkv,
-                         int D, int P, float scale, int window) {
+                         int D, int P, float scale, int window, const float* head_scale, float softcap,
+                         int keep_first, int sink) {
     const size_t floats = (size_t)QR * D + (size_t)WAVES * QR * 64 + WAVES * 64 + WAVES * QR * 2 +
                           (size_t)WAVES * QR * D;
     dim3 grid((T_tokens + QR - 1) / QR, Hq), block(WAVES * 64);
     hipLaunchKernelGGL((attn_plain_kernel<T, QR, WAVES>), grid, block, floats * sizeof(float), st, (const T*)q,
                        (T*)out, (const T*)k_pool, (const T*)v_pool, page_table, cu_pages, kv_start, cu_q,
-                       q_start, tok_ids, n_seqs, T_tokens, Hq, Hkv, D, P, scale, window);
+                       q_start, tok_ids, n_seqs, T_tokens, Hq, Hkv, D, P, scale, window, head_scale, softcap,
+                       keep_first, sink);
 }
 
 extern "C" int ra_attention_plain(const void* q, void* out, const void* k_pool, const void* v_pool,
                                   const int* page_table, const int* cu_pages, const int* kv_start,
                                   const int* cu_q, const int* q_start, const int* tok_ids,
                                   int n_seqs, int T_tokens, int Hq, int Hkv, int D, int P, float scale, int window, int dtype,
-                                  void* stream) {
+                                  const float* head_scale, float softcap, int keep_first, int sink, void* stream) {
     if (T_tokens <= 0 || n_seqs <= 0) return RA_OK;
     if (D > 64 * PLAIN_MAX_ACC || D <= 0 || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 || Hq > 65535) return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
@@ -274,7 +292,8 @@ extern "C" int ra_attention_plain(const void* q, void* out, const void* k_pool, 
     const bool single = tok_ids == nullptr && T_tokens == n_seqs;
 #define PLAIN_GO(T_, QR_, W_)                                                                              \
     plain_launch<T_, QR_, W_>(st, q, out, k_pool, v_pool, page_table, cu_pages, kv_start, cu_q, q_start,   \
-                              tok_ids, n_seqs, T_tokens, Hq, Hkv, D, P, scale, window)
+                              tok_ids, n_seqs, T_tokens, Hq, Hkv, D, P, scale, window, head_scale, softcap,   \
+                              keep_first, sink)
     if (dtype == RA_DTYPE_F32) {
         if (single) PLAIN_GO(float, 1, 8); else PLAIN_GO(float, 4, 4);
     } else {

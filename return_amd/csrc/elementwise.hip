@@ -3,6 +3,7 @@
 // Formulas: rollout/fused.py:6-17 (RMSNorm), rollout/attention.py:10-25 (rotation),
 // rollout/fused.py:103-114 (SiLU-mul), rollout/cache.py:334-337 (cache write).
 #include "common.h"
+#include <algorithm>
 
 // ------------------------------------------------------------------ embedding
 template <typename T>
@@ -744,5 +745,131 @@ extern "C" int ra_silu_mul(const void* gu, void* out, int T_tokens, int I, int d
     else
         hipLaunchKernelGGL(silu_mul_kernel<bf16>, grid, block, 0, (hipStream_t)stream,
                            (const bf16*)gu, (bf16*)out, I, total);
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ squared ReLU, in place
+// x <- max(x, 0)^2 over n elements.
+template <typename T>
+__global__ void relu_sq_kernel(T* __restrict__ x, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        const float v = fmaxf(to_f(x[i]), 0.f);
+        x[i] = from_f<T>(v * v);
+    }
+}
+
+extern "C" int ra_relu_sq(void* x, long long n, int dtype, void* stream) {
+    if (n <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)std::min<long long>((n + 255) / 256, 65536));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(relu_sq_kernel<float>, grid, block, 0, (hipStream_t)stream, (float*)x, (size_t)n);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(relu_sq_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (bf16*)x, (size_t)n);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ bias over rows, in place
+// x [rows, N] += b [N] (b in 32-bit).
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ b, int N, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) x[i] = from_f<T>(to_f(x[i]) + b[i % N]);
+}
+
+extern "C" int ra_add_bias(void* x, const float* b, long long rows, int N, int dtype, void* stream) {
+    const long long n = rows * N;
+    if (n <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)std::min<long long>((n + 255) / 256, 65536));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(add_bias_kernel<float>, grid, block, 0, (hipStream_t)stream, (float*)x, b, N, (size_t)n);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(add_bias_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (bf16*)x, b, N, (size_t)n);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ q/k preparation where the values are the keys
+// One wave per (token, head) over the projection row [q heads | k heads]: an optional bias (32-bit,
+// one entry per column) is added, the first R elements of the head rotate by the token's position
+// (pairs (j, j + R/2)), q goes to q_out [T, Hq, D], the rotated k to its row of the key pool and the
+// k as projected (with its bias, before the rotation) to the same row of the value pool.
+template <typename T>
+__global__ void qk_prepare_kernel(const T* __restrict__ qk, int Hq, int Hkv, int D, const float* __restrict__ bias,
+                                  const int* __restrict__ positions, const float* __restrict__ cos_t,
+                                  const float* __restrict__ sin_t, int R, T* __restrict__ q_out,
+                                  T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ slots,
+                                  int P, long long pool_rows, long long n_rows) {
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const int heads = Hq + Hkv;
+    const int t = (int)(row / heads);
+    const int head = (int)(row % heads);
+    const T* src = qk + row * D;
+    const float* b = bias ? bias + (size_t)head * D : nullptr;
+    T* dst;
+    T* plain = nullptr;
+    if (head < Hq) {
+        dst = q_out + ((size_t)t * Hq + head) * D;
+    } else {
+        if (k_pool == nullptr) return;
+        const long long s = slots[t];
+        if (s < 0 || s >= pool_rows) return;
+        const size_t at = ra_cache_offset(s, head - Hq, Hkv, P, D);
+        dst = k_pool + at;
+        plain = v_pool + at;
+    }
+    const int half = R >> 1;
+    const int pos = positions[t];
+    for (int j = lane; j < half; j += 64) {
+        float x1 = to_f(src[j]), x2 = to_f(src[j + half]);
+        if (b) {
+            x1 += b[j];
+            x2 += b[j + half];
+        }
+        const float cs = cos_t[(size_t)pos * half + j], sn = sin_t[(size_t)pos * half + j];
+        if (plain) {
+            plain[j] = from_f<T>(x1);
+            plain[j + half] = from_f<T>(x2);
+            // the key that rotates is the stored one: what the value pool holds, rotated
+            x1 = round_to<T>(x1);
+            x2 = round_to<T>(x2);
+        }
+        dst[j] = from_f<T>(x1 * cs - x2 * sn);
+        dst[j + half] = from_f<T>(x2 * cs + x1 * sn);
+    }
+    for (int c = R + lane; c < D; c += 64) {
+        float x = to_f(src[c]);
+        if (b) x += b[c];
+        dst[c] = from_f<T>(x);
+        if (plain) plain[c] = from_f<T>(x);
+    }
+}
+
+extern "C" int ra_qk_prepare(const void* qk, int T_tokens, int Hq, int Hkv, int D, const float* bias,
+                             const int* positions, const float* cos_t, const float* sin_t, int R, void* q_out,
+                             void* k_pool, void* v_pool, const int* slots, int P, long long pool_rows, int dtype,
+                             void* stream) {
+    if (T_tokens <= 0) return RA_OK;
+    if ((k_pool == nullptr) != (v_pool == nullptr) || (k_pool != nullptr && P <= 0)) return RA_ERR_ARG;
+    if (D < 1 || R < 0 || R > D || (R & 1)) return RA_ERR_ARG;
+    const long long n_rows = (long long)T_tokens * (Hq + Hkv);
+    dim3 block(256), grid((unsigned)((n_rows + 3) / 4));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(qk_prepare_kernel<float>, grid, block, 0, (hipStream_t)stream, (const float*)qk, Hq, Hkv, D,
+                           bias, positions, cos_t, sin_t, R, (float*)q_out, (float*)k_pool, (float*)v_pool, slots, P,
+                           pool_rows, n_rows);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(qk_prepare_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (const bf16*)qk, Hq, Hkv, D,
+                           bias, positions, cos_t, sin_t, R, (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, P,
+                           pool_rows, n_rows);
+    else
+        return RA_ERR_ARG;
     return ra_launch_status();
 }

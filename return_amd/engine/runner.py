@@ -53,6 +53,7 @@ class ModelRunner:
         _, build_spec = lookup_architecture(config.architecture)
         self.spec = build_spec(config)
         self.rt = Runtime(ec.device, ec.dtype, ops=ops)
+        self.rt.position_limit = int(ec.max_token)      # no request holds more tokens than the pool has rows
         if hasattr(self.rt.ops, "defer_norms"):
             self.rt.ops.defer_norms = bool(ec.defer_norms)
         if weights is None:
@@ -73,7 +74,7 @@ class ModelRunner:
         self.builder = StepBuilder(self.cache, ec.max_step_tokens, ec.max_reside, self.rt.device,
                                    tile_rows=needs["prefill_tile_rows"], token_columns=needs["token_columns"])
         self.vocab_size = self.spec.vocab_size
-        self.max_position = self.spec.max_position
+        self.max_position = self.spec.max_position if self.spec.max_position is not None else int(ec.max_token)
         # decode-only steps replayed from captured HIP graphs (rollout/model.py:346-407 captures one
         # graph per batch size; here one per (batch size, context bucket))
         self._graphs = {}

@@ -70,7 +70,14 @@ def _declare(lib):
         "ra_gemm_sweep_fits": [I, I],
         "ra_gemm_sweep_workgroups": [I, I],
         "ra_gemm_sweep_norm_bf16": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P],
-        "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, F, I, I, P],
+        "ra_causal_conv": [P, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
+        "ra_delta_rule": [P, L, P, L, I, I, I, I, I, P, P, P, P, P, F, P, P, P, P, I, I, I, I, I, I, P],
+        "ra_delta_rule_fits": [I, I, I, I],
+        "ra_token_side": [P, P, P, P, L, I, P, P, P, F, I, I, I, I, P],
+        "ra_relu_sq": [P, L, I, P],
+        "ra_add_bias": [P, P, L, I, I, P],
+        "ra_qk_prepare": [P, I, I, I, I, P, P, P, P, I, P, P, P, P, I, L, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, I, P],
         "ra_attention_decode_static_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
@@ -357,6 +364,147 @@ class HipOps:
             raise KernelError(f"silu_mul: gate-up {tuple(gu.shape)}, out {tuple(out.shape)}")
         self._check(self.lib.ra_silu_mul(_ptr(gu), _ptr(out), T, I, _code(gu.dtype), self._stream()),
                     "silu_mul")
+
+    # ------------------------------------------------------------------ parts beside the usual ones
+    def _want_rows(self, t, name, dtype=None):
+        """A matrix whose rows may be a column slice of a wider one: rows apart by stride(0), elements side by side."""
+        if t.device != self.device:
+            raise KernelError(f"{name} is on {t.device}, kernels run on {self.device}")
+        if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1) or (t.shape[0] > 1 and t.stride(0) < t.shape[1]):
+            raise KernelError(f"{name} must be rows of elements side by side, got shape {tuple(t.shape)} strides {t.stride()}")
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError(f"{name} must be {dtype}, got {t.dtype}")
+        return t.stride(0) if t.shape[0] > 1 else max(t.shape[1], t.stride(0))
+
+    def relu_sq(self, x):
+        """x <- max(x, 0)^2 in place."""
+        self._want(x, "activations")
+        self._check(self.lib.ra_relu_sq(_ptr(x), x.numel(), _code(x.dtype), self._stream()), "relu_sq")
+        return x
+
+    def add_bias(self, x, bias):
+        """x [rows, N] += bias [N] (32-bit) in place."""
+        self._want(x, "rows", dims=2)
+        self._want(bias, "bias", torch.float32, 1)
+        if bias.shape[0] != x.shape[1]:
+            raise KernelError(f"add_bias: rows {tuple(x.shape)}, bias {tuple(bias.shape)}")
+        self._check(self.lib.ra_add_bias(_ptr(x), _ptr(bias), x.shape[0], x.shape[1], _code(x.dtype), self._stream()),
+                    "add_bias")
+        return x
+
+    def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False):
+        """out = act(conv(x)) or act(x + conv(x)): a causal convolution over time on each channel, the last
+        taps-1 inputs of every request kept in tail [slots, taps-1, C] between steps (rows by the step's
+        slot_ids). x: [T, C], possibly a column slice of wider rows; w: fp32 [C, taps], last column the
+        current row's; out: [T, C] rows, not x."""
+        ld_x = self._want_rows(x, "conv input")
+        ld_out = self._want_rows(out, "conv output", x.dtype)
+        self._want(w, "conv weight", torch.float32, 2)
+        self._want(tail, "conv tail", x.dtype, 3)
+        T, C = x.shape
+        taps = w.shape[1]
+        if tuple(out.shape) != (T, C) or w.shape[0] != C or tuple(tail.shape[1:]) != (taps - 1, C) or T != step.n_tokens:
+            raise KernelError(f"causal_conv: x {tuple(x.shape)}, w {tuple(w.shape)}, tail {tuple(tail.shape)}, "
+                              f"out {tuple(out.shape)}, step of {step.n_tokens}")
+        if not 1 <= taps <= 8:
+            raise KernelError(f"causal_conv: {taps} taps, the kernel takes 1 to 8")
+        if max(step.slot_ids_host, default=0) >= tail.shape[0]:
+            raise KernelError("causal_conv: a request's slot lies beyond the tail's rows")
+        if out.data_ptr() == x.data_ptr():
+            raise KernelError("causal_conv: the output must not be the input")
+        self._check(self.lib.ra_causal_conv(
+            _ptr(x), ld_x, _ptr(w), _ptr(tail), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(out), ld_out, step.n_seqs,
+            step.max_q_len, C, taps, (1 if add_input else 0) | (2 if silu else 0), _code(x.dtype), self._stream()),
+            "causal_conv")
+        return out
+
+    def delta_rule_fits(self, D, V, rank_a, rank_g):
+        return bool(self.lib.ra_delta_rule_fits(int(D), int(V), int(rank_a), int(rank_g)))
+
+    def delta_rule(self, qkv, z, off_b, off_a, rank_a, off_g, rank_g, w_a2t, w_g2t, a_log, dt_bias, norm_w, eps,
+                   state, step, out, H, G, D, V):
+        """The gated delta rule with a decay per key channel over the step's rows, with everything around it
+        (unit q and k, beta, the decay's and the output gate's low-rank second factors, the norm of the
+        read-out) in the one kernel. qkv: [T, 2 G D + H V] after the short convolution; z: the fused input
+        projection's rows (beta at column off_b, the low-rank first factors at off_a and off_g);
+        state: fp32 [slots, H, D, V], updated in place; out: [T, H V]."""
+        ld_qkv = self._want_rows(qkv, "delta-rule q/k/v")
+        ld_z = self._want_rows(z, "delta-rule projections", qkv.dtype)
+        self._want(out, "delta-rule output", qkv.dtype, 2)
+        self._want(state, "delta-rule state", torch.float32, 4)
+        T = qkv.shape[0]
+        for t, name, shape in ((w_a2t, "decay factor", (rank_a, H * D)), (w_g2t, "gate factor", (rank_g, H * V)),
+                               (a_log, "A_log", (H,)), (dt_bias, "dt_bias", (H * D,)), (norm_w, "norm weight", (V,))):
+            self._want(t, name, torch.float32)
+            if tuple(t.shape) != shape:
+                raise KernelError(f"delta_rule: {name} is {tuple(t.shape)}, wanted {shape}")
+        if qkv.shape[1] != 2 * G * D + H * V or tuple(out.shape) != (T, H * V) or z.shape[0] != T or T != step.n_tokens \
+                or tuple(state.shape[1:]) != (H, D, V) or H % G:
+            raise KernelError(f"delta_rule: qkv {tuple(qkv.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)}, "
+                              f"state {tuple(state.shape)}, {H} heads over {G} of {D} x {V}, step of {step.n_tokens}")
+        if max(off_b + H, off_a + rank_a, off_g + rank_g) > z.shape[1] or min(off_b, off_a, off_g) < 0:
+            raise KernelError(f"delta_rule: columns {off_b}, {off_a}, {off_g} beyond rows of {z.shape[1]}")
+        if max(step.slot_ids_host, default=0) >= state.shape[0]:
+            raise KernelError("delta_rule: a request's slot lies beyond the state's rows")
+        if not self.delta_rule_fits(D, V, rank_a, rank_g):
+            raise KernelError(f"delta_rule: heads of {D} x {V} with ranks {rank_a}, {rank_g} are beyond the kernel")
+        self._check(self.lib.ra_delta_rule(
+            _ptr(qkv), ld_qkv, _ptr(z), ld_z, off_b, off_a, rank_a, off_g, rank_g, _ptr(w_a2t), _ptr(w_g2t), _ptr(a_log),
+            _ptr(dt_bias), _ptr(norm_w), float(eps), _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(out),
+            step.n_seqs, H, G, D, V, _code(qkv.dtype), self._stream()), "delta_rule")
+        return out
+
+    def token_side(self, h, delta, token_ids, table, offset, gate, proj, weight, eps):
+        """h += delta, then h += rmsnorm(proj (gelu_tanh(gate h) * table[token][offset:offset+S])) * weight,
+        row by row, in place. delta may be None."""
+        self._want(h, "residual stream", torch.float32, 2)
+        T, H = h.shape
+        self._want(token_ids, "token ids", torch.int32, 1)
+        self._want(gate, "side gate", dims=2)
+        S = gate.shape[0]
+        self._want(proj, "side projection", gate.dtype, 2)
+        self._want(table, "side table", gate.dtype, 2)
+        self._want(weight, "side norm weight", torch.float32, 1)
+        if delta is not None:
+            self._want(delta, "delta", gate.dtype, 2)
+        if tuple(gate.shape) != (S, H) or tuple(proj.shape) != (H, S) or weight.shape[0] != H or token_ids.shape[0] != T \
+                or (delta is not None and tuple(delta.shape) != (T, H)) or offset < 0 or offset + S > table.shape[1]:
+            raise KernelError(f"token_side: h {tuple(h.shape)}, gate {tuple(gate.shape)}, proj {tuple(proj.shape)}, "
+                              f"table {tuple(table.shape)} at {offset}")
+        if S > 64 or H > 8192:
+            raise KernelError(f"token_side: {S} side channels (at most 64) for rows of {H} (at most 8192)")
+        self._check(self.lib.ra_token_side(_ptr(h), _ptr(delta), _ptr(token_ids), _ptr(table), table.shape[1], int(offset),
+                                           _ptr(gate), _ptr(proj), _ptr(weight), float(eps), T, H, S,
+                                           _code(gate.dtype), self._stream()), "token_side")
+
+    def qk_prepare(self, qk, n_q, n_kv, D, bias, positions, cos, sin, rotary_dim, q_out, k_pool, v_pool, slot_mapping):
+        """q/k preparation of an attention whose values are its keys as projected: bias, rotation of the first
+        rotary_dim elements, q to q_out, the rotated k to the key pool and the unrotated k to the value pool."""
+        self._want(qk, "qk", dims=2)
+        self._want(q_out, "q", qk.dtype, 3)
+        self._want(positions, "positions", torch.int32, 1)
+        self._want(slot_mapping, "slot mapping", torch.int32, 1)
+        T = qk.shape[0]
+        R = int(rotary_dim)
+        if qk.shape[1] != (n_q + n_kv) * D or tuple(q_out.shape) != (T, n_q, D) or positions.shape[0] != T \
+                or slot_mapping.shape[0] != T:
+            raise KernelError(f"qk_prepare: qk {tuple(qk.shape)}, q {tuple(q_out.shape)}, {T} tokens")
+        if bias is not None:
+            self._want(bias, "bias", torch.float32, 1)
+            if bias.shape[0] != qk.shape[1]:
+                raise KernelError(f"qk_prepare: bias {tuple(bias.shape)} for rows of {qk.shape[1]}")
+        if R:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if R % 2 or R > D or cos.shape[1] != R // 2 or sin.shape != cos.shape:
+                raise KernelError(f"qk_prepare: rotary_dim {R}, tables {tuple(cos.shape)}, head size {D}")
+        rows = 0
+        if k_pool is not None:
+            rows = self._pool_rows(k_pool, v_pool, n_kv, D, qk.dtype)
+        self._check(self.lib.ra_qk_prepare(
+            _ptr(qk), T, n_q, n_kv, D, _ptr(bias), _ptr(positions), _ptr(cos) if R else None, _ptr(sin) if R else None, R,
+            _ptr(q_out), _ptr(k_pool), _ptr(v_pool), _ptr(slot_mapping), k_pool.shape[2] if k_pool is not None else 0,
+            rows, _code(qk.dtype), self._stream()), "qk_prepare")
 
     # ------------------------------------------------------------------ matrix products
     # Ways to form y = x @ w^T from bfloat16 operands. Which is fastest depends on the shape in ways no
@@ -781,7 +929,11 @@ class HipOps:
             return (rows,) if rows == 64 else (rows, 64)
         return None
 
-    def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
+    def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0, head_scale=None, softcap=0.0,
+                  keep_first=0, sink=False):
+        """Attention of the step's queries over the paged cache. Optional: head_scale (fp32, one factor per query
+        head on the scale), softcap c (score -> c tanh(score / c)), keep_first n (keys at positions below n
+        stay visible whatever the window), sink (one more key of score 0 without a value in the softmax)."""
         self._want(q, "q", dims=3)
         self._want(out, "attention output", q.dtype, 3)
         T, n_q, D = q.shape
@@ -796,9 +948,15 @@ class HipOps:
         P = k_pool.shape[2]
         window = int(window)
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
-        fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
+        softcap, keep_first, sink = float(softcap or 0.0), int(keep_first or 0), bool(sink)
+        if head_scale is not None:
+            self._want(head_scale, "head scale", torch.float32, 1)
+            if head_scale.shape[0] != n_q:
+                raise KernelError(f"attention: head scale {tuple(head_scale.shape)} for {n_q} heads")
+        plain_only = head_scale is not None or softcap > 0.0 or keep_first > 0 or sink
+        fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256 and not plain_only
         fast_prefill = q.dtype == torch.bfloat16 and bool(step.prefill_tiles) and D % 16 == 0 and D <= 256 and \
-            (fast_decode or step.n_decode == 0)
+            (fast_decode or step.n_decode == 0) and not plain_only
 
         def decode_part():
             S, max_splits, merge = self._decode_splits(step, n_q, n_kv, D, window)
@@ -863,7 +1021,8 @@ class HipOps:
             return
         self._check(self.lib.ra_attention_plain(
             _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
-            n_q, n_kv, D, P, float(scale), window, _code(q.dtype), self._stream()), "attention_plain")
+            n_q, n_kv, D, P, float(scale), window, _code(q.dtype), _ptr(head_scale), softcap, keep_first,
+            1 if sink else 0, self._stream()), "attention_plain")
 
     def _decode_splits(self, step, n_q, n_kv, D, window):
         """Keys per split of the decode attention, the most splits a request has, and whether a

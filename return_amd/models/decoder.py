@@ -98,7 +98,13 @@ class Decoder:
         """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
         h = self.embedding.forward(step.token_ids, step)
         pending = None
+        h_in = h.clone() if any(call.add_input for call in self.schedule) else None
         for i, call in enumerate(self.schedule):
+            if call.add_input:
+                if pending is not None:                   # what the part before left goes into the stream first
+                    self.rt.ops.residual_add(h, pending)
+                    pending = None
+                self.rt.ops.residual_add(h, h_in)
             view = None
             if call.cache is not None:
                 view = tuple(cache.view(c) for c in call.cache) if isinstance(call.cache, (tuple, list)) \

@@ -11,6 +11,18 @@ un-rotated in the pool; here K is rotated once when it is written, which gives t
 same scores because a request's positions never change.
 Scale is D^-0.5 unless given (rollout/attention.py:195). Query head h reads kv head
 h // (Hq/Hkv) (rollout/attention.py:65).
+
+Beyond the reference, each off unless its parameter is given:
+  values "keys"        there is no value projection: a token's value is its key as projected (with its
+                       bias), before the rotation. The key pool holds the rotated keys, the value pool the
+                       unrotated ones.
+  bias True            q, k (and v, where there is one) and the output projection have biases
+                       (roles q_bias, k_bias, v_bias, o_bias), added in the projection
+  head_temperature     a learned factor per query head on the scale (role "temp", [Hq])
+  softcap c            score <- c tanh(score / c), after scale and temperature
+  window w, keep_first n   position i reads j <= i with i - j < w or j < n; the first n keys keep
+                       their true positions
+  sink True            softmax with one added to the denominator: a key of score 0 that has no value
 """
 from __future__ import annotations
 
@@ -27,6 +39,14 @@ class PagedAttention:
                          params["head_dim"])
         shapes = {"q_proj": (Hq * D, H), "k_proj": (Hkv * D, H), "v_proj": (Hkv * D, H),
                   "o_proj": (H, Hq * D)}
+        if params.get("values", "projected") == "keys":
+            del shapes["v_proj"]
+        if params.get("bias"):
+            shapes.update({"q_bias": (Hq * D,), "k_bias": (Hkv * D,), "o_bias": (H,)})
+            if "v_proj" in shapes:
+                shapes["v_bias"] = (Hkv * D,)
+        if params.get("head_temperature"):
+            shapes["temp"] = (Hq,)
         if params.get("qk_norm_eps") is not None:
             shapes["q_norm"] = (D,)
             shapes["k_norm"] = (D,)
@@ -34,7 +54,9 @@ class PagedAttention:
 
     @staticmethod
     def random_init(params, role):
-        return "norm" if role in ("q_norm", "k_norm") else "matrix"
+        if role in ("q_norm", "k_norm", "temp"):
+            return "norm"
+        return "matrix"
 
     def __init__(self, params, tensors, rt, shared=None):
         self.rt = rt
@@ -52,19 +74,35 @@ class PagedAttention:
         self.position = (shared or {}).get(params["position"]) if params.get("position") else None
         if params.get("position") and self.position is None:
             raise KeyError(f"attention names position encoding {params['position']!r}, which the model lacks")
-        self.w_qkv = rt.product(torch.cat([rt.matrix(tensors["q_proj"]), rt.matrix(tensors["k_proj"]),
-                                           rt.matrix(tensors["v_proj"])], dim=0).contiguous())
-        self.w_o = rt.product(rt.matrix(tensors["o_proj"]), residual=True)
+        self.values_are_keys = params.get("values", "projected") == "keys"
+        self.keep_first = int(params.get("keep_first") or 0)
+        self.softcap = float(params.get("softcap") or 0.0)
+        self.sink = bool(params.get("sink"))
+        self.temp = rt.vector32(tensors["temp"]) if params.get("head_temperature") else None
+        self.extras = {}
+        if self.temp is not None or self.softcap or self.keep_first or self.sink:
+            self.extras = dict(head_scale=self.temp, softcap=self.softcap, keep_first=self.keep_first, sink=self.sink)
+        self.bias_in = self.bias_o = None
+        names = ("q_proj", "k_proj") if self.values_are_keys else ("q_proj", "k_proj", "v_proj")
+        if params.get("bias"):
+            self.bias_in = torch.cat([rt.vector32(tensors[n[0] + "_bias"]) for n in names]).contiguous()
+            self.bias_o = rt.vector32(tensors["o_bias"])
+            if not self.values_are_keys:
+                raise ValueError("attention: biases are built for the form whose values are its keys only")
+        if self.values_are_keys and self.eps is not None:
+            raise ValueError("attention: per-head norms are not built for the form whose values are its keys")
+        self.w_qkv = rt.product(torch.cat([rt.matrix(tensors[n]) for n in names], dim=0).contiguous())
+        self.w_o = rt.product(rt.matrix(tensors["o_proj"]), residual=self.bias_o is None)
         self.w_qn = rt.vector32(tensors["q_norm"]) if self.eps is not None else None
         self.w_kn = rt.vector32(tensors["k_norm"]) if self.eps is not None else None
-        self._fusable = self.position is None or hasattr(self.position, "tables")
+        self._fusable = (self.position is None or hasattr(self.position, "tables")) and not self.values_are_keys
         # x goes into one product only and the output comes out of one: a norm before may be left to
         # the first (ScaledRows as x), a norm after may be finished inside the second (sink)
         self.first_product = (self.w_qkv, False)
-        self.last_product = self.w_o
+        self.last_product = self.w_o if self.bias_o is None else None
 
     def cache_spec(self):
-        return PagedKVSpec(self.n_kv, self.d, self.window)
+        return PagedKVSpec(self.n_kv, self.d, self.window, self.keep_first)
 
     def step_needs(self):
         """The q-tile list that the kernel set's attention reads for requests with more than one token."""
@@ -78,7 +116,20 @@ class PagedAttention:
         T, Hq, Hkv, D = x.shape[0], self.n_q, self.n_kv, self.d
         tables = step.groups[cache.group]
         qkv = ops.linear(x, self.w_qkv)                              # [T, (Hq+2Hkv)*D]
-        if self._fusable and write_cache and hasattr(ops, "attention_qkv"):
+        if self.values_are_keys:
+            if self.position is not None and not hasattr(self.position, "tables"):
+                raise ValueError("attention whose values are its keys rotates by tables only")
+            cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
+            q = rt.empty(T, Hq, D)
+            ops.qk_prepare(qkv, Hq, Hkv, D, self.bias_in, step.positions, cos, sin, rot, q,
+                           cache.k_pool if write_cache else None, cache.v_pool if write_cache else None,
+                           tables.slot_mapping)
+            o = rt.empty(T, Hq, D)
+            ops.attention(q, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale,
+                          int(self.window) if self.window else 0, **self.extras)
+            y = project(o.view(T, Hq * D), self.w_o)
+            return ops.add_bias(y, self.bias_o) if self.bias_o is not None else y
+        if self._fusable and not self.extras and write_cache and hasattr(ops, "attention_qkv"):
             # every request brings one token: the kernel set may prepare q, k and v inside its attention
             cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
             o = rt.empty(T, Hq, D)
@@ -111,7 +162,7 @@ class PagedAttention:
                 ops.kv_write(k, v, cache.k_pool, cache.v_pool, tables.slot_mapping)
         o = rt.empty(T, Hq, D)
         ops.attention(q, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale,
-                      int(self.window) if self.window else 0)
+                      int(self.window) if self.window else 0, **self.extras)
         return project(o.view(T, Hq * D), self.w_o)
 
 

@@ -99,7 +99,64 @@ class PreNormBlock:
         return h, f
 
 
-BLOCKS = {"pre_norm": PreNormBlock}
+class ConvSideBlock:
+    """Pre-norm layer with a causal convolution in front of every sublayer and a token input at its end:
+
+        h += mixer(conv_m(norm_m(h)));  h += feed_forward(conv_f(norm_f(h)));  h += token_input(h, token)
+
+    where conv(x) = x + filter(x) over time (an "input_conv" part). Parts by name: mixer_norm, mixer and,
+    each optional, mixer_conv, feed_forward_norm + feed_forward (both or neither), feed_forward_conv,
+    token_input. What the layer keeps between steps is what its mixer keeps plus, if it has
+    convolutions, one state of their tails: cache_spec() is the tuple (mixer's spec(s)..., tails)."""
+
+    def __init__(self, spec, build):
+        has = lambda name: name in spec.parts
+        self.mixer_norm = build("mixer_norm")
+        self.mixer = build("mixer")
+        self.mixer_conv = build("mixer_conv") if has("mixer_conv") else None
+        self.feed_forward = build("feed_forward") if has("feed_forward") else None
+        self.feed_forward_norm = build("feed_forward_norm") if self.feed_forward is not None else None
+        self.feed_forward_conv = build("feed_forward_conv") if has("feed_forward_conv") and self.feed_forward is not None \
+            else None
+        self.token_input = build("token_input") if has("token_input") else None
+        mixer_spec = self.mixer.cache_spec()
+        self._mixer_specs = () if mixer_spec is None else \
+            tuple(mixer_spec) if isinstance(mixer_spec, (tuple, list)) else (mixer_spec,)
+        tails = []
+        for name, conv in (("mixer_tail", self.mixer_conv), ("feed_forward_tail", self.feed_forward_conv)):
+            if conv is not None:
+                tails.append((name, tuple(conv.state_shape()), conv.rt.dtype_name))
+        from ..cache.spec import StateSpec
+        self._tails = StateSpec(tuple(tails)) if tails else None
+
+    def cache_spec(self):
+        specs = self._mixer_specs + ((self._tails,) if self._tails is not None else ())
+        return None if not specs else specs[0] if len(specs) == 1 else specs
+
+    def step_needs(self):
+        return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
+
+    def forward(self, h, pending, step, cache, write_cache=True):
+        views = () if cache is None else tuple(cache) if isinstance(cache, (tuple, list)) else (cache,)
+        n = len(self._mixer_specs)
+        mixer_cache = None if n == 0 else views[0] if n == 1 else views[:n]
+        tails = views[n].tensors if self._tails is not None else None
+        x = self.mixer_norm.forward(h, pending)
+        if self.mixer_conv is not None:
+            x = self.mixer_conv.forward(x, step, tails["mixer_tail"])
+        pending = self.mixer.forward(x, step, mixer_cache, write_cache)
+        if self.feed_forward is not None:
+            x = self.feed_forward_norm.forward(h, pending)
+            if self.feed_forward_conv is not None:
+                x = self.feed_forward_conv.forward(x, step, tails["feed_forward_tail"])
+            pending = self.feed_forward.forward(x, step)
+        if self.token_input is not None:
+            self.token_input.forward(h, pending, step)
+            pending = None
+        return h, pending
+
+
+BLOCKS = {"pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock}
 
 
 def register_arrangement(name, cls):

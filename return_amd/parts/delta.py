@@ -1,0 +1,110 @@
+"""Gated delta rule with a decay per key channel: a mixer whose memory is a matrix S [D, V] per head,
+of fixed size whatever the sequence's length.
+
+For head h with its q/k head h // (heads / kv_heads), token by token:
+    q, k, v    = silu(short causal conv(W_q x)), ... (one filter per channel, taps from the config)
+    q, k       <- unit vectors per head, x / sqrt(sum x^2 + 1e-6); q also times D^-1/2
+    beta       = sigmoid(W_b x)                                   one per head
+    g          = exp(-exp(A_log[h]) * softplus(W_a2 (W_a1 x) + dt_bias))    one per head and key channel
+    S          <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+    y          = W_o (o / rms(o) * w_norm * sigmoid(W_g2 (W_g1 x)))        rms over the head's V, w_norm [V]
+Everything from the unit vectors to the norm of o is 32-bit. Kept between steps per request: the
+last taps-1 inputs of the three convolutions and S.
+
+One product forms q, k, v, b and the first factors of the two low-rank maps (the weights stacked,
+rows padded to a multiple of 16); the convolution reads its columns of that result in place; the
+recurrence kernel reads the rest and applies the second factors itself.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..cache.spec import StateSpec
+from .conv import filter_init
+from .registry import register_part
+
+DEFAULT_RANK = 16
+
+
+def _a_log_init(shape, generator):
+    """Logarithm of a decay rate: log of U(0.02, 1)."""
+    return torch.log(0.02 + 0.98 * torch.rand(*shape, generator=generator, dtype=torch.float32, device=generator.device))
+
+
+def _dt_bias_init(shape, generator):
+    """Bias of the decay's step size: U(-4, -1), so that softplus starts small and the memory long."""
+    return -4.0 + 3.0 * torch.rand(*shape, generator=generator, dtype=torch.float32, device=generator.device)
+
+
+class ChannelDeltaMixer:
+    @staticmethod
+    def tensor_shapes(params):
+        W, H, G, D, V = (params["hidden_size"], params["num_heads"], params["num_kv_heads"], params["head_dim"],
+                         params["value_dim"])
+        taps = params["conv_taps"]
+        ra, rg = params.get("decay_rank"), params.get("gate_rank")      # None: whatever the stored tensor has
+        return {"q_proj": (G * D, W), "k_proj": (G * D, W), "v_proj": (H * V, W),
+                "q_conv": (G * D, taps), "k_conv": (G * D, taps), "v_conv": (H * V, taps),
+                "b_proj": (H, W), "A_log": (H,), "dt_bias": (H * D,), "o_norm": (V,),
+                "a1_proj": (ra, W), "a2_proj": (H * D, ra), "g1_proj": (rg, W), "g2_proj": (H * V, rg),
+                "o_proj": (W, H * V)}
+
+    @staticmethod
+    def random_init(params, role):
+        if role in ("q_conv", "k_conv", "v_conv"):
+            return filter_init
+        return {"A_log": _a_log_init, "dt_bias": _dt_bias_init, "o_norm": "norm"}.get(role, "matrix")
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.hidden = W = int(params["hidden_size"])
+        self.H, self.G = int(params["num_heads"]), int(params["num_kv_heads"])
+        self.D, self.V = int(params["head_dim"]), int(params["value_dim"])
+        self.taps = int(params["conv_taps"])
+        self.eps = float(params["eps"])
+        if self.H % self.G:
+            raise ValueError(f"{self.H} heads are not a multiple of {self.G} q/k heads")
+        self.ra, self.rg = tensors["a1_proj"].shape[0], tensors["g1_proj"].shape[0]
+        if tensors["a2_proj"].shape[1] != self.ra or tensors["g2_proj"].shape[1] != self.rg:
+            raise ValueError("the two factors of a low-rank map differ in their inner size")
+        if hasattr(rt.ops, "delta_rule_fits") and not rt.ops.delta_rule_fits(self.D, self.V, self.ra, self.rg):
+            raise ValueError(f"heads of {self.D} x {self.V} with low-rank maps of {self.ra} and {self.rg} are beyond "
+                             "the delta-rule kernel")
+        self.c_conv = 2 * self.G * self.D + self.H * self.V
+        self.off_b = self.c_conv
+        self.off_a = self.off_b + self.H
+        self.off_g = self.off_a + self.ra
+        used = self.off_g + self.rg
+        rows = [rt.matrix(tensors[n]) for n in ("q_proj", "k_proj", "v_proj", "b_proj", "a1_proj", "g1_proj")]
+        pad = -used % 16
+        if pad:
+            rows.append(torch.zeros(pad, W, dtype=rt.dtype, device=rt.device))
+        self.w_in = rt.product(torch.cat(rows, dim=0).contiguous())
+        self.w_conv = torch.cat([rt.vector32(tensors[n]) for n in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
+        self.w_a2t = rt.vector32(tensors["a2_proj"]).t().contiguous()          # [ra, H*D]
+        self.w_g2t = rt.vector32(tensors["g2_proj"]).t().contiguous()          # [rg, H*V]
+        self.a_log = rt.vector32(tensors["A_log"])
+        self.dt_bias = rt.vector32(tensors["dt_bias"])
+        self.w_norm = rt.vector32(tensors["o_norm"])
+        self.w_o = rt.product(rt.matrix(tensors["o_proj"]))
+
+    def cache_spec(self):
+        return StateSpec((("conv", (self.taps - 1, self.c_conv), self.rt.dtype_name),
+                          ("S", (self.H, self.D, self.V), "float32")))
+
+    def forward(self, x, step, cache, write_cache=True):
+        rt, ops = self.rt, self.rt.ops
+        if not write_cache:
+            raise ValueError("a delta-rule mixer advances its state with every call; it cannot only read it")
+        T = x.shape[0]
+        z = ops.linear(x, self.w_in)                                           # [T, q | k | v | b | a1 | g1 | pad]
+        qkv = rt.empty(T, self.c_conv)
+        ops.causal_conv(z[:, :self.c_conv], self.w_conv, cache.tensors["conv"], step, qkv, silu=True)
+        o = rt.empty(T, self.H * self.V)
+        ops.delta_rule(qkv, z, self.off_b, self.off_a, self.ra, self.off_g, self.rg, self.w_a2t, self.w_g2t,
+                       self.a_log, self.dt_bias, self.w_norm, self.eps, cache.tensors["S"], step, o,
+                       self.H, self.G, self.D, self.V)
+        return ops.linear(o, self.w_o)
+
+
+register_part("mixer", "channel_delta", ChannelDeltaMixer)

@@ -36,3 +36,28 @@ class SwiGLU:
 
 
 register_part("feed_forward", "swiglu", SwiGLU)
+
+
+class SquaredReLU:
+    """Dense feed-forward down(relu(up(x))^2), no biases."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        H, I = params["hidden_size"], params["intermediate_size"]
+        return {"up_proj": (I, H), "down_proj": (H, I)}
+
+    @staticmethod
+    def random_init(params, role):
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.w_up = rt.product(rt.matrix(tensors["up_proj"]))
+        self.w_down = rt.product(rt.matrix(tensors["down_proj"]))
+
+    def forward(self, x, step=None):
+        ops = self.rt.ops
+        return ops.linear(ops.relu_sq(ops.linear(x, self.w_up)), self.w_down)
+
+
+register_part("feed_forward", "relu2", SquaredReLU)

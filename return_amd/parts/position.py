@@ -22,16 +22,25 @@ class RotaryPosition:
         self.head_dim = int(params["head_dim"])
         self.rotary_dim = int(params.get("rotary_dim", self.head_dim))
         self.theta = float(params["theta"])
-        self.max_position = int(params["max_position"])
+        # no limit of the model's own: as many positions as the engine's cache can hold for one request
+        limit = params.get("max_position")
+        self.max_position = int(limit if limit is not None else getattr(rt, "position_limit", 0) or 0)
+        if self.max_position < 1:
+            raise ValueError("rotary positions: neither the model nor the engine says how many positions there are")
         self.scaling = float(params.get("attention_scaling", 1.0))
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
         self.rt = rt
         half = self.rotary_dim // 2
-        inv_freq = 1.0 / (self.theta ** (torch.arange(0, half, dtype=torch.float32) / half))
-        angle = torch.outer(torch.arange(self.max_position, dtype=torch.float32), inv_freq)
-        self.cos = (angle.cos() * self.scaling).to(rt.device).contiguous()
-        self.sin = (angle.sin() * self.scaling).to(rt.device).contiguous()
+        if params.get("exact_tables"):
+            # frequencies and angles in 64-bit, so that the 32-bit tables are the rounded true values
+            inv_freq = self.theta ** (-torch.arange(0, half, dtype=torch.float64) / half)
+            angle = torch.outer(torch.arange(self.max_position, dtype=torch.float64), inv_freq)
+        else:
+            inv_freq = 1.0 / (self.theta ** (torch.arange(0, half, dtype=torch.float32) / half))
+            angle = torch.outer(torch.arange(self.max_position, dtype=torch.float32), inv_freq)
+        self.cos = (angle.cos() * self.scaling).float().to(rt.device).contiguous()
+        self.sin = (angle.sin() * self.scaling).float().to(rt.device).contiguous()
 
     def tables(self):
         """(cos, sin, rotary_dim): fp32 [max_position, rotary_dim/2] each."""

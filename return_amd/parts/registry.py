@@ -46,6 +46,11 @@ Interfaces (``rt`` is the return_amd.parts.runtime.Runtime of the engine):
                 int32 [T] (what a request brings with its tokens, StepEntry.columns / Engine.submit's
                 token_columns; the position where it brings nothing), and apply is called as
                 apply(q, k, positions, step). Mixers and embeddings may declare columns the same way.
+  input_conv    a filter over time in front of a sublayer, whose last inputs the block keeps between steps:
+                state_shape() -> (rows, channels) of the tail it needs per request;
+                forward(x, step, tail) -> x + conv(x)   tail: [slots, rows, channels], updated in place
+  token_input   something a layer adds to the stream for the token itself, after its other parts:
+                forward(h, pending, step)   h += pending (if any), then h += f(h, step.token_ids), in place
   embedding     forward(token_ids, step) -> h  fp32 [T, H]   (step.positions for absolute positions)
   head          forward(x) -> logits fp32 [rows, V]
 """
@@ -53,7 +58,7 @@ from __future__ import annotations
 
 from typing import Dict
 
-CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head")
+CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "input_conv", "token_input")
 _PARTS: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
 
 

@@ -93,6 +93,8 @@ class Runtime:
             ops = HipOps(self.device)
         self.ops = ops
         self._cast: Dict[int, torch.Tensor] = {}
+        self.position_limit = None          # most positions a request can reach (the engine's cache size), for parts
+                                            # of a model that sets no limit of its own
         self.products = []                  # (weight, gated, result dtype) of the parts' matrix products
         self.norm_pairs = []                # (weight before, norm weight, eps, weight after, gated) of norms between two products
 

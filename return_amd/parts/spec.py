@@ -56,10 +56,14 @@ class LayerCall:
             tuple of numbers, one for each spec of a block whose cache_spec() is a tuple.
             Two calls may name the same cache layer; only calls with writes_cache=True
             append to it, the others read what an earlier call wrote in the same step.
+    add_input: the embedding's output (the stream as it was before the first call) is added to
+            the stream right before this call, as a looped stack does at the start of every pass
+            but its first.
     """
     block: int
     cache: Optional[object] = None
     writes_cache: bool = True
+    add_input: bool = False
 
 
 @dataclasses.dataclass
@@ -67,7 +71,7 @@ class ModelSpec:
     architecture: str
     hidden_size: int
     vocab_size: int
-    max_position: int
+    max_position: Optional[int]         # None: the design sets no limit (the cache's size is the limit)
     embedding: PartSpec
     positions: Dict[str, PartSpec]      # named position encodings that mixers refer to
     blocks: List[BlockSpec]

@@ -76,8 +76,10 @@ def load_weights(folder: str, spec: ModelSpec, device="cpu") -> Dict[str, torch.
                 shapes[name] = tuple(f.get_slice(name).get_shape())
     missing = sorted(n for n in expected if n not in found)
     unexpected = sorted(n for n in found if n not in expected and n not in ignorable)
+    # (None in an expected shape: that size is whatever the stored tensor has; the part reads it there)
+    fits = lambda got, want: len(got) == len(want) and all(w is None or g == w for g, w in zip(got, want))
     misshaped = sorted((n, shapes[n], expected[n][0]) for n in expected
-                       if n in found and shapes[n] != tuple(expected[n][0]))
+                       if n in found and not fits(shapes[n], tuple(expected[n][0])))
     if missing or unexpected or misshaped:
         raise WeightError(folder, missing, unexpected, misshaped)
     out: Dict[str, torch.Tensor] = {}

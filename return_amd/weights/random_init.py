@@ -37,6 +37,9 @@ def random_weights(spec, seed: int = 0, std: float = 0.02, embedding_std: Option
     expected = spec.expected_tensors()
     for name in sorted(expected):
         shape, draw = expected[name]
+        if any(d is None for d in shape):
+            raise ValueError(f"{name}: the model leaves a size of this tensor to the stored weights {tuple(shape)}; "
+                             "random weights need it in the configuration")
         if callable(draw):
             # the part's own law, drawn from the same generator (so the seed still fixes the model)
             x = draw(tuple(shape), gen)

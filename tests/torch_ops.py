@@ -142,7 +142,8 @@ class TorchOps:
 
     # rollout/attention.py:126-139 over the tables of rollout/cache.py:282-328,
     # gathered as opd/test_parallel.py:14-42 does
-    def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0):
+    def attention(self, q, out, k_pool, v_pool, step, group, scale, window=0, head_scale=None, softcap=0.0,
+                  keep_first=0, sink=False):
         g = step.groups[group]
         n_q, n_kv = q.shape[1], k_pool.shape[1]
         cu_q, cu_p = step.cu_q.tolist(), g.cu_pages.tolist()
@@ -159,11 +160,110 @@ class TorchOps:
             kk = k.repeat_interleave(n_q // n_kv, dim=1)
             vv = v.repeat_interleave(n_q // n_kv, dim=1)
             score = torch.einsum("qhd,khd->hqk", q[a:b].float(), kk) * scale
+            if head_scale is not None:
+                score = score * head_scale.float()[:, None, None]
+            if softcap:
+                score = softcap * torch.tanh(score / softcap)
             hide = k_pos[None, :] > q_pos[:, None]
             if window:
-                hide = hide | (k_pos[None, :] <= q_pos[:, None] - window)
+                far = k_pos[None, :] <= q_pos[:, None] - window
+                if keep_first:
+                    far = far & (k_pos[None, :] >= keep_first)
+                hide = hide | far
             score = score.masked_fill(hide[None], float("-inf"))
-            out[a:b] = torch.einsum("hqk,khd->qhd", score.softmax(-1), vv).to(out.dtype)
+            if sink:                                        # one more key of score 0 that has no value
+                zero = torch.zeros_like(score[..., :1])
+                prob = torch.cat([score, zero], dim=-1).softmax(-1)[..., :-1]
+            else:
+                prob = score.softmax(-1)
+            out[a:b] = torch.einsum("hqk,khd->qhd", prob, vv).to(out.dtype)
+
+    # ---- the parts beside the usual ones, each as its kernel is called
+    def relu_sq(self, x):
+        x.copy_((torch.relu(x.float()) ** 2).to(x.dtype))
+        return x
+
+    def add_bias(self, x, bias):
+        x.copy_((x.float() + bias).to(x.dtype))
+        return x
+
+    def causal_conv(self, x, w, tail, step, out, add_input=False, silu=False):
+        taps = w.shape[1]
+        cu, slots = step.cu_q_host, step.slot_ids_host
+        for s in range(step.n_seqs):
+            a, b = cu[s], cu[s + 1]
+            seq = torch.cat([tail[slots[s]].float(), x[a:b].float()], dim=0)       # [taps-1 + n, C]
+            y = torch.zeros(b - a, x.shape[1], dtype=torch.float32, device=x.device)
+            for j in range(taps):
+                y += w[:, j] * seq[j:j + (b - a)]
+            if add_input:
+                y = y + x[a:b].float()
+            if silu:
+                y = y * torch.sigmoid(y)
+            out[a:b] = y.to(out.dtype)
+            if taps > 1:
+                tail[slots[s]] = seq[-(taps - 1):].to(tail.dtype)
+        return out
+
+    def delta_rule_fits(self, D, V, rank_a, rank_g):
+        return True
+
+    def delta_rule(self, qkv, z, off_b, off_a, rank_a, off_g, rank_g, w_a2t, w_g2t, a_log, dt_bias, norm_w, eps,
+                   state, step, out, H, G, D, V):
+        cu, slots = step.cu_q_host, step.slot_ids_host
+        T = qkv.shape[0]
+        q = qkv[:, :G * D].float().view(T, G, D)
+        k = qkv[:, G * D:2 * G * D].float().view(T, G, D)
+        v = qkv[:, 2 * G * D:].float().view(T, H, V)
+        q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
+        k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+        beta = torch.sigmoid(z[:, off_b:off_b + H].float())
+        a = z[:, off_a:off_a + rank_a].float() @ w_a2t + dt_bias
+        g = torch.exp(-torch.exp(a_log)[None, :, None] * torch.nn.functional.softplus(a).view(T, H, D))
+        gate = torch.sigmoid(z[:, off_g:off_g + rank_g].float() @ w_g2t).view(T, H, V)
+        rep = H // G
+        for s in range(step.n_seqs):
+            S = state[slots[s]]                               # [H, D, V], updated in place
+            for t in range(cu[s], cu[s + 1]):
+                kt, qt = k[t].repeat_interleave(rep, 0), q[t].repeat_interleave(rep, 0)    # [H, D]
+                S *= g[t][:, :, None]
+                u = beta[t][:, None] * (v[t] - torch.einsum("hdv,hd->hv", S, kt))
+                S += kt[:, :, None] * u[:, None, :]
+                o = torch.einsum("hdv,hd->hv", S, qt)
+                o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * norm_w * gate[t]
+                out[t] = o.reshape(-1).to(out.dtype)
+        return out
+
+    def token_side(self, h, delta, token_ids, table, offset, gate, proj, weight, eps):
+        if delta is not None:
+            h += delta.float()
+        S = gate.shape[0]
+        e = table[token_ids.long()][:, offset:offset + S].float()
+        a = h @ gate.float().t()
+        g = 0.5 * a * (1 + torch.tanh(0.7978845608028654 * (a + 0.044715 * a ** 3))) * e
+        y = g @ proj.float().t()
+        h += y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * weight
+
+    def qk_prepare(self, qk, n_q, n_kv, D, bias, positions, cos, sin, rotary_dim, q_out, k_pool, v_pool, slot_mapping):
+        T = qk.shape[0]
+        x = qk.float()
+        if bias is not None:
+            x = x + bias
+        q = x[:, :n_q * D].reshape(T, n_q, D)
+        k = x[:, n_q * D:].reshape(T, n_kv, D).to(qk.dtype)     # the value pool's rows; the keys are these, rotated
+
+        def rot(x):
+            if not rotary_dim:
+                return x
+            half = rotary_dim // 2
+            c = cos[positions.long()][:, None, :]
+            s = sin[positions.long()][:, None, :]
+            x1, x2 = x[..., :half], x[..., half:rotary_dim]
+            return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s, x[..., rotary_dim:]], dim=-1)
+
+        q_out.copy_(rot(q).to(q_out.dtype))
+        if k_pool is not None:
+            self.kv_write(rot(k.float()).to(qk.dtype), k, k_pool, v_pool, slot_mapping)
 
     # rollout/model.py:15-61 with the draw made by inverse CDF in vocabulary order
     def sample(self, logits, temperature, top_k, top_p, u):
