@@ -7,11 +7,11 @@
 //     h_t[c] += y[c] / sqrt(mean_c y[c]^2 + eps) * w[c]
 // gelu_tanh(x) = 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))). Sums, the norm and the stream are
 // 32-bit; gate [S, H], proj [H, S] and the table [vocab, ld_table] are in the storage type.
-// One workgroup per row: every thread sums its columns' share of the S gate products, the shares are
-// added over the workgroup through LDS, then every thread forms its columns of y.
+// One workgroup per row: every thread sums its columns' share of the gate products (SB of them a pass), the
+// shares are added over the workgroup through LDS, then every thread forms its columns of y.
 #include "common.h"
 
-#define TS_MAX_S 64
+#define TS_MAX_S 512
 #define TS_THREADS 256
 #define TS_MAX_CPT 32        // columns per thread: H <= 256 * 32
 
@@ -21,37 +21,39 @@ __global__ __launch_bounds__(TS_THREADS) void token_side_kernel(
     long long ld_table, int off, const T* __restrict__ gate, const T* __restrict__ proj, const float* __restrict__ w,
     float eps, int H, int S) {
     __shared__ float part[TS_THREADS / 64][SB];
-    __shared__ float g_s[SB];
+    __shared__ float g_s[TS_MAX_S];
     __shared__ float red[16];
     const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float* hr = h + (size_t)t * H;
-    float a[SB];
+    for (int r0 = 0; r0 < S; r0 += SB) {                 // SB gate rows a pass; the first pass adds delta into the stream
+        float a[SB];
 #pragma unroll
-    for (int r = 0; r < SB; ++r) a[r] = 0.f;
-    for (int c = tid; c < H; c += TS_THREADS) {
-        float v = hr[c];
-        if (delta != nullptr) {
-            v += to_f(delta[(size_t)t * H + c]);
-            hr[c] = v;
+        for (int r = 0; r < SB; ++r) a[r] = 0.f;
+        for (int c = tid; c < H; c += TS_THREADS) {
+            float v = hr[c];
+            if (r0 == 0 && delta != nullptr) {
+                v += to_f(delta[(size_t)t * H + c]);
+                hr[c] = v;                               // (read again by this thread only)
+            }
+#pragma unroll
+            for (int r = 0; r < SB; ++r)
+                if (r0 + r < S) a[r] = fmaf(to_f(gate[(size_t)(r0 + r) * H + c]), v, a[r]);
         }
 #pragma unroll
-        for (int r = 0; r < SB; ++r)
-            if (r < S) a[r] = fmaf(to_f(gate[(size_t)r * H + c]), v, a[r]);
+        for (int r = 0; r < SB; ++r) {
+            const float v = wave_sum(a[r]);
+            if (lane == 0) part[wave][r] = v;
+        }
+        __syncthreads();
+        if (tid < SB && r0 + tid < S) {
+            float x = 0.f;
+            for (int wv = 0; wv < TS_THREADS / 64; ++wv) x += part[wv][tid];
+            const float inner = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+            const float e = to_f(table[(size_t)ids[t] * ld_table + off + r0 + tid]);
+            g_s[r0 + tid] = 0.5f * x * (1.f + tanhf(inner)) * e;
+        }
+        __syncthreads();
     }
-#pragma unroll
-    for (int r = 0; r < SB; ++r) {
-        const float v = wave_sum(a[r]);
-        if (lane == 0) part[wave][r] = v;
-    }
-    __syncthreads();
-    if (tid < S) {
-        float x = 0.f;
-        for (int wv = 0; wv < TS_THREADS / 64; ++wv) x += part[wv][tid];
-        const float inner = 0.7978845608028654f * (x + 0.044715f * x * x * x);
-        const float e = to_f(table[(size_t)ids[t] * ld_table + off + tid]);
-        g_s[tid] = 0.5f * x * (1.f + tanhf(inner)) * e;
-    }
-    __syncthreads();
     float y[TS_MAX_CPT];
     float ss = 0.f;
 #pragma unroll

@@ -471,8 +471,8 @@ class HipOps:
                 or (delta is not None and tuple(delta.shape) != (T, H)) or offset < 0 or offset + S > table.shape[1]:
             raise KernelError(f"token_side: h {tuple(h.shape)}, gate {tuple(gate.shape)}, proj {tuple(proj.shape)}, "
                               f"table {tuple(table.shape)} at {offset}")
-        if S > 64 or H > 8192:
-            raise KernelError(f"token_side: {S} side channels (at most 64) for rows of {H} (at most 8192)")
+        if S > 512 or H > 8192:
+            raise KernelError(f"token_side: {S} side channels (at most 512) for rows of {H} (at most 8192)")
         self._check(self.lib.ra_token_side(_ptr(h), _ptr(delta), _ptr(token_ids), _ptr(table), table.shape[1], int(offset),
                                            _ptr(gate), _ptr(proj), _ptr(weight), float(eps), T, H, S,
                                            _code(gate.dtype), self._stream()), "token_side")

@@ -62,7 +62,7 @@ def test_causal_conv(ops, ref, dtype, C, taps, q_lens, flags):
     the input is a column slice of wider rows."""
     add_input, silu = flags
     n = len(q_lens)
-    slots = [(3 * i + 1) % (n + 2) for i in range(n)]
+    slots = torch.randperm(n + 2, generator=torch.Generator().manual_seed(n)).tolist()[:n]
     w = rnd(C, taps, seed=1, scale=0.5)
     tail_a = rnd(n + 2, taps - 1, C, dtype=dtype, seed=2)
     tail_b = tail_a.clone()
@@ -86,7 +86,7 @@ def test_causal_conv(ops, ref, dtype, C, taps, q_lens, flags):
 def test_delta_rule(ops, ref, dtype, H, G, D, V, ra, rg, q_lens):
     n = len(q_lens)
     T = sum(q_lens)
-    slots = [(2 * i + 1) % (n + 1) for i in range(n)]
+    slots = torch.randperm(n + 1, generator=torch.Generator().manual_seed(n)).tolist()[:n]
     qkv = rnd(T, 2 * G * D + H * V, dtype=dtype, seed=1)
     z = rnd(T, 16 + H + ra + rg + 5, dtype=dtype, seed=2)
     w_a2t, w_g2t = rnd(ra, H * D, seed=3, scale=0.5), rnd(rg, H * V, seed=4, scale=0.5)
@@ -235,8 +235,15 @@ def test_attention_one_key_decides(ops, dtype, q_len, where):
 
 # ------------------------------------------------------------------ the engine against the plain model
 LENGTHS = {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 150, "g": 1, "h": 47}
-# largest differences seen on these traces: 2e-5 in 32-bit, 0.05 in bfloat16 on logits of up to 4
-TOL = {"float32": dict(atol=2e-4, rtol=1e-4), "bfloat16": dict(atol=0.15, rtol=5e-2)}
+# A row's error: the root mean square over the vocabulary of the difference of the logits, its mean taken off,
+# over the root mean square of the plain logits. 32-bit: ten times the largest seen on these traces (3e-6).
+# bfloat16: what rounding alone does differs from row to row by a factor of ten (a stand-in engine of torch
+# operations that rounds where the kernels round is 0.01 to 0.14 away from the plain logits on the very rows
+# on which the kernels are), so the kernels are held against that stand-in, row by row (twice the largest
+# difference seen, 0.013), and against the plain logits on average and by a bound that only a fault exceeds.
+ROW_ERROR = {"float32": 5e-5, "bfloat16": 0.3}
+ROW_ERROR_16_MEAN = 0.03
+ROW_ERROR_16_STAND_IN = 0.03
 
 
 @pytest.fixture(scope="module", params=sorted(CASES))
@@ -244,36 +251,52 @@ def model(request, tmp_path_factory):
     folder = make_folder(tmp_path_factory, request.param)
     cfg, w = plain.read_folder(folder)
     reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in LENGTHS.items()}
-    return folder, cfg, reqs, {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    # the same requests, whole, through the engine with torch operations in bfloat16 in place of the kernels
+    steps = tt.whole(reqs)
+    rounded = tt.run_in_process(make_runner(folder, "bfloat16", tt.peak_tokens(steps), ops=TorchOps(DEV)), steps)
+    return folder, cfg, reqs, want, rounded
 
 
-def make_runner(folder, dtype, max_tokens, page=16, **kw):
+def make_runner(folder, dtype, max_tokens, page=16, ops=None, **kw):
     from return_amd.config import EngineConfig
     from return_amd.engine import ModelRunner
     ec = EngineConfig(dtype=dtype, page_size=page, max_token=max_tokens, max_reside=4, max_step_tokens=max(max_tokens, 4),
                       prefill_chunk=max_tokens, tune_products=False, check_invariants=True, **kw)
-    return ModelRunner(folder, engine_config=ec)
+    return ModelRunner(folder, engine_config=ec, ops=ops)
 
 
-def compare(got, want, reqs, dtype):
-    worst = 0.0
+def row_error(a, b):
+    d = (a - b).double()
+    return float((d - d.mean()).pow(2).mean().sqrt() / b.double().pow(2).mean().sqrt())
+
+
+def compare(got, want, reqs, dtype, rounded=None):
+    worst, total, n = 0.0, 0.0, 0
     for rid, toks in reqs.items():
         for p in range(len(toks)):
-            a, b = got[(rid, p)], want[rid][p]
-            worst = max(worst, (a - b).abs().max().item())
-            torch.testing.assert_close(a, b, **TOL[dtype],
-                                       msg=lambda m: f"request {rid} position {p} (first wrong place): {m}")
+            e = row_error(got[(rid, p)], want[rid][p])
+            worst, total, n = max(worst, e), total + e, n + 1
+            assert e <= ROW_ERROR[dtype], f"request {rid} position {p} (first wrong place): row error {e:.3e}"
+            if dtype == "float32":
+                assert int(got[(rid, p)].argmax()) == int(want[rid][p].argmax()), f"request {rid} position {p}: argmax"
+            elif rounded is not None:
+                e16 = row_error(got[(rid, p)], rounded[(rid, p)])
+                assert e16 <= ROW_ERROR_16_STAND_IN, \
+                    f"request {rid} position {p} (first wrong place): {e16:.3e} from the stand-in that rounds alike"
+    if dtype == "bfloat16":
+        assert total / n <= ROW_ERROR_16_MEAN, f"mean row error {total / n:.3e}"
     return worst
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("cut", ["whole", "tail_decoded", "portions", "mixed"])
 def test_engine_matches_plain(model, dtype, cut):
-    folder, cfg, reqs, want = model
+    folder, cfg, reqs, want, rounded = model
     steps = {"whole": tt.whole, "tail_decoded": tt.tail_decoded, "portions": tt.portions, "mixed": tt.mixed}[cut](reqs)
     runner = make_runner(folder, dtype, tt.peak_tokens(steps))
     got = tt.run_in_process(runner, steps)
-    print(f"kofipel {dtype} {cut}: largest difference {compare(got, want, reqs, dtype):.2e}")
+    print(f"kofipel {dtype} {cut}: largest row error {compare(got, want, reqs, dtype, rounded):.2e}")
     assert not runner.cache.live and all(g.pages.in_use() == 0 for g in runner.cache.groups)
 
 
@@ -286,11 +309,12 @@ def test_long_decoding_passes_the_window(tmp_path_factory, dtype):
     toks = tt.random_tokens(cfg["vocab"], 300, seed=4)
     steps = tt.tail_decoded({"r": toks}, tail=280)
     got = tt.run_in_process(make_runner(folder, dtype, 320), steps)
-    compare(got, {"r": plain.logits(cfg, w, toks)}, {"r": toks}, dtype)
+    print(f"kofipel {dtype} long decoding: largest row error {compare(got, {'r': plain.logits(cfg, w, toks)}, {'r': toks}, dtype):.2e}")
 
 
 def test_batches_of_unequal_requests_equal_each_alone(tmp_path_factory):
-    """Bit for bit in 32-bit: a request's logits do not depend on what else is in the step."""
+    """A request's logits do not depend on what else is in the step, beyond the rounding of products that
+    the library forms in another order for another number of rows."""
     folder = make_folder(tmp_path_factory, "b")
     cfg, _ = plain.read_folder(folder)
     reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in (("a", 70), ("b", 3), ("c", 41), ("d", 1))}
@@ -312,7 +336,7 @@ def test_batches_of_unequal_requests_equal_each_alone(tmp_path_factory):
         steps.append({"step": k, "entries": entries, "end": end})
     together = tt.run_in_process(make_runner(folder, "float32", 256), steps)
     for key, row in alone.items():
-        torch.testing.assert_close(together[key], row, atol=1e-5, rtol=1e-5)
+        assert row_error(together[key], row) < 2e-5
 
 
 # ------------------------------------------------------------------ generation and the programs
