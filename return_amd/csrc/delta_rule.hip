@@ -15,7 +15,8 @@
 //
 // A workgroup takes one (head, request) and walks the request's rows in chunks of DR_TC: first
 // everything that does not depend on S is prepared for the chunk in LDS by all threads (the decay's
-// low-rank map, softplus, exponentials, the unit vectors), then the recurrence runs over the chunk
+// low-rank map, whose second factor's rows for this head are copied into LDS once when they fit,
+// softplus, exponentials, the unit vectors), then the recurrence runs over the chunk
 // without a barrier, then the chunk's read-outs are normed, gated and stored. In the recurrence a
 // column j of S belongs to RS neighbouring lanes, each with DPT rows in registers; the two sums
 // over rows are finished by lane swaps.
@@ -27,13 +28,26 @@
 __device__ __forceinline__ float dr_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float dr_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
+// Sum over the RS (1, 2, 4 or 8) neighbouring lanes that share a column, in every one of them, by
+// data-parallel moves inside a row of 16 lanes: partner lane ^ 1, then lane ^ 2, then the other quad
+// of the eight (mirrored: after the first two steps a quad's lanes all hold the quad's sum).
+__device__ __forceinline__ float dr_group_sum(float v, int RS) {
+    if (RS >= 2)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    if (RS >= 4)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    if (RS >= 8)
+        v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    return v;
+}
+
 template <typename T, int DPT>
 __global__ __launch_bounds__(512) void delta_rule_kernel(
     const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ z, long long ld_z, int off_b, int off_a,
     int ra, int off_g, int rg, const float* __restrict__ w_a2t, const float* __restrict__ w_g2t,
     const float* __restrict__ A_log, const float* __restrict__ dt_bias, const float* __restrict__ norm_w,
     float eps, float* __restrict__ S, const int* __restrict__ cu_q, const int* __restrict__ slot_ids,
-    T* __restrict__ out, int H, int G, int D, int V, int RS) {
+    T* __restrict__ out, int H, int G, int D, int V, int RS, int staged) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int tid = threadIdx.x, NT = blockDim.x, lane = tid & 63, wave = tid >> 6, n_waves = NT >> 6;
     const int h = blockIdx.x, s = blockIdx.y, kvh = h / (H / G);
@@ -49,6 +63,19 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     float* a1_s = o_s + DR_TC * V;                  // [TC][ra]
     float* g1_s = a1_s + DR_TC * ra;                // [TC][rg]
     float* beta_s = g1_s + DR_TC * rg;              // [TC]
+    // staged: this head's rows of the two low-rank second factors sit in LDS for the whole walk
+    float* wa_s = beta_s + DR_TC;                   // [ra][D]
+    float* wg_s = wa_s + (staged ? ra * D : 0);     // [rg][V]
+    if (staged) {
+        for (int idx = tid; idx < ra * D; idx += NT) {
+            const int r = idx / D, i = idx - r * D;
+            wa_s[idx] = w_a2t[(size_t)r * H * D + h * D + i];
+        }
+        for (int idx = tid; idx < rg * V; idx += NT) {
+            const int r = idx / V, jj = idx - r * V;
+            wg_s[idx] = w_g2t[(size_t)r * H * V + h * V + jj];
+        }
+    }
 
     const int j = tid / RS, rp = tid % RS;
     const bool live = j < V;
@@ -89,7 +116,11 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
                 qq = to_f(row[kvh * D + i]);
                 kk = to_f(row[G * D + kvh * D + i]);
                 float a = dt_bias[h * D + i];
-                for (int r = 0; r < ra; ++r) a = fmaf(a1_s[tt * ra + r], w_a2t[(size_t)r * H * D + h * D + i], a);
+                if (staged) {
+                    for (int r = 0; r < ra; ++r) a = fmaf(a1_s[tt * ra + r], wa_s[r * D + i], a);
+                } else {
+                    for (int r = 0; r < ra; ++r) a = fmaf(a1_s[tt * ra + r], w_a2t[(size_t)r * H * D + h * D + i], a);
+                }
                 gg = expf(neg_a * dr_softplus(a));
             }
             k_s[at] = kk;
@@ -119,21 +150,21 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
             const float* qr = q_s + tt * DP + rp * PS;
             const float* gr = g_s + tt * DP + rp * PS;
             float kreg[DPT];
-            float acc = 0.f;
+            float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;         // four chains, so that no sum waits for the one before
 #pragma unroll
             for (int ii = 0; ii < DPT; ii += 4) {
                 const float4 k4 = *reinterpret_cast<const float4*>(kr + ii);
                 const float4 g4 = *reinterpret_cast<const float4*>(gr + ii);
                 kreg[ii] = k4.x; kreg[ii + 1] = k4.y; kreg[ii + 2] = k4.z; kreg[ii + 3] = k4.w;
                 st[ii] *= g4.x; st[ii + 1] *= g4.y; st[ii + 2] *= g4.z; st[ii + 3] *= g4.w;
-                acc = fmaf(st[ii], k4.x, acc);
-                acc = fmaf(st[ii + 1], k4.y, acc);
-                acc = fmaf(st[ii + 2], k4.z, acc);
-                acc = fmaf(st[ii + 3], k4.w, acc);
+                a0 = fmaf(st[ii], k4.x, a0);
+                a1 = fmaf(st[ii + 1], k4.y, a1);
+                a2 = fmaf(st[ii + 2], k4.z, a2);
+                a3 = fmaf(st[ii + 3], k4.w, a3);
             }
-            for (int m = 1; m < RS; m <<= 1) acc += __shfl_xor(acc, m, 64);
+            const float acc = dr_group_sum((a0 + a1) + (a2 + a3), RS);
             const float u = beta_s[tt] * (v_s[tt * V + (live ? j : 0)] - acc);
-            float o = 0.f;
+            float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DPT; ii += 4) {
                 const float4 q4 = *reinterpret_cast<const float4*>(qr + ii);
@@ -141,12 +172,12 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
                 st[ii + 1] = fmaf(kreg[ii + 1], u, st[ii + 1]);
                 st[ii + 2] = fmaf(kreg[ii + 2], u, st[ii + 2]);
                 st[ii + 3] = fmaf(kreg[ii + 3], u, st[ii + 3]);
-                o = fmaf(st[ii], q4.x, o);
-                o = fmaf(st[ii + 1], q4.y, o);
-                o = fmaf(st[ii + 2], q4.z, o);
-                o = fmaf(st[ii + 3], q4.w, o);
+                o0 = fmaf(st[ii], q4.x, o0);
+                o1 = fmaf(st[ii + 1], q4.y, o1);
+                o2 = fmaf(st[ii + 2], q4.z, o2);
+                o3 = fmaf(st[ii + 3], q4.w, o3);
             }
-            for (int m = 1; m < RS; m <<= 1) o += __shfl_xor(o, m, 64);
+            const float o = dr_group_sum((o0 + o1) + (o2 + o3), RS);
             if (live && rp == 0) o_s[tt * V + j] = o;
         }
         __syncthreads();
@@ -157,7 +188,11 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
             const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
             for (int jj = lane; jj < V; jj += 64) {
                 float gate = 0.f;
-                for (int r = 0; r < rg; ++r) gate = fmaf(g1_s[tt * rg + r], w_g2t[(size_t)r * H * V + h * V + jj], gate);
+                if (staged) {
+                    for (int r = 0; r < rg; ++r) gate = fmaf(g1_s[tt * rg + r], wg_s[r * V + jj], gate);
+                } else {
+                    for (int r = 0; r < rg; ++r) gate = fmaf(g1_s[tt * rg + r], w_g2t[(size_t)r * H * V + h * V + jj], gate);
+                }
                 out[(size_t)(base + c0 + tt) * H * V + h * V + jj] =
                     from_f<T>(o_s[tt * V + jj] * rstd * norm_w[jj] * dr_sigmoid(gate));
             }
@@ -174,6 +209,9 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
 static size_t delta_rule_lds(int DPT, int RS, int V, int ra, int rg) {
     return sizeof(float) * ((size_t)DR_TC * (3 * RS * (DPT + DR_PAD) + 2 * V + ra + rg) + DR_TC);
 }
+// the low-rank factors' rows of one head beside that, if they fit
+static size_t delta_rule_staged(int D, int V, int ra, int rg) { return sizeof(float) * ((size_t)ra * D + (size_t)rg * V); }
+#define DR_LDS_LIMIT (156 * 1024)
 
 // The split of a column's rows over lanes: RS lanes (a power of two) of DPT rows each.
 static bool delta_rule_plan(int D, int V, int* RS_out, int* DPT_out) {
@@ -200,7 +238,7 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
                              const void* z, long long ld_z, int off_b, int off_a, int ra, int off_g, int rg,
                              const float* w_a2t, const float* w_g2t, const float* A_log, const float* dt_bias,
                              const float* norm_w, float eps, float* S, const int* cu_q, const int* slot_ids, void* out,
-                             int H, int G, int D, int V, int RS) {
+                             int H, int G, int D, int V, int RS, int staged) {
 #define DR_GO(DPT_)                                                                                               \
     do {                                                                                                          \
         if (lds > 64 * 1024 &&                                                                                    \
@@ -209,7 +247,7 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
             return RA_ERR_LAUNCH;                                                                                 \
         hipLaunchKernelGGL((delta_rule_kernel<T, DPT_>), grid, block, lds, st, (const T*)qkv, ld_qkv, (const T*)z, \
                            ld_z, off_b, off_a, ra, off_g, rg, w_a2t, w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q,  \
-                           slot_ids, (T*)out, H, G, D, V, RS);                                                    \
+                           slot_ids, (T*)out, H, G, D, V, RS, staged);                                            \
     } while (0)
     switch (DPT) {
         case 4: DR_GO(4); break;
@@ -233,15 +271,17 @@ extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* z, l
     if (!delta_rule_plan(D, V, &RS, &DPT) || H < 1 || G < 1 || H % G || ra < 0 || rg < 0 || n_seqs > 65535) return RA_ERR_ARG;
     if (ld_qkv < (long long)2 * G * D + (long long)H * V || off_b < 0 || off_a < 0 || off_g < 0) return RA_ERR_ARG;
     if (ld_z < off_b + H || ld_z < off_a + ra || ld_z < off_g + rg) return RA_ERR_ARG;
-    const size_t lds = delta_rule_lds(DPT, RS, V, ra, rg);
+    size_t lds = delta_rule_lds(DPT, RS, V, ra, rg);
     if (lds > 160 * 1024) return RA_ERR_ARG;
+    const int staged = lds + delta_rule_staged(D, V, ra, rg) <= DR_LDS_LIMIT ? 1 : 0;
+    if (staged) lds += delta_rule_staged(D, V, ra, rg);
     dim3 grid(H, n_seqs), block(((V * RS + 63) / 64) * 64);
     hipStream_t st = (hipStream_t)stream;
     if (dtype == RA_DTYPE_F32)
         return delta_rule_launch<float>(st, DPT, grid, block, lds, qkv, ld_qkv, z, ld_z, off_b, off_a, ra, off_g, rg, w_a2t,
-                                        w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids, out, H, G, D, V, RS);
+                                        w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids, out, H, G, D, V, RS, staged);
     if (dtype == RA_DTYPE_BF16)
         return delta_rule_launch<bf16>(st, DPT, grid, block, lds, qkv, ld_qkv, z, ld_z, off_b, off_a, ra, off_g, rg, w_a2t,
-                                       w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids, out, H, G, D, V, RS);
+                                       w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids, out, H, G, D, V, RS, staged);
     return RA_ERR_ARG;
 }

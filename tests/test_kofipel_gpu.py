@@ -106,7 +106,8 @@ def test_delta_rule(ops, ref, dtype, H, G, D, V, ra, rg, q_lens):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,H,S,with_delta", [(1, 72, 5, True), (7, 256, 24, False), (3, 4096, 64, True),
-                                              (40, 1000, 17, True), (2, 8192, 33, False), (5, 64, 100, True)])
+                                              (40, 1000, 17, True), (2, 8192, 33, False), (5, 64, 100, True),
+                                              (301, 512, 16, True), (258, 4096, 32, False)])
 def test_token_side(ops, ref, dtype, T, H, S, with_delta):
     table = rnd(50, 3 * S + 1, dtype=dtype, seed=1)
     gate, proj = rnd(S, H, dtype=dtype, seed=2, scale=H ** -0.5), rnd(H, S, dtype=dtype, seed=3)
