@@ -52,14 +52,19 @@ typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
 
 typedef short4_t __attribute__((address_space(3))) * lds_short4_ptr;
 
-template <int D16, int QG, int KSPLIT>
+// XT: the optional extras. head_scale[h] multiplies the scale of query head h; softcap c turns a score s
+// into c tanh(s / c); keys at positions below keep_first stay readable whatever the window (their tiles
+// are walked first, then the tiles from the window's first key on); sink adds one to the softmax's
+// denominator (a key of score 0 that has no value).
+template <int D16, int QG, int KSPLIT, bool XT>
 __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ page_table,
     const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ tiles,       // [n_tiles][2]: request number, first row of the tile within it
-    int n_tiles, int Hq, int Hkv, int P, float scale, int window) {
+    int n_tiles, int Hq, int Hkv, int P, float scale, int window,
+    const float* __restrict__ head_scale, float softcap, int keep_first, int sink) {
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;
     constexpr bool TAIL16 = (D % 32) != 0;
@@ -139,8 +144,29 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
     const int tile_last_pos = pos0 + min(q_off + BM, q_len) - 1;
     int first_key = start;
     if (window > 0 && tile_first_pos - window + 1 > first_key) first_key = tile_first_pos - window + 1;
+    // The key tiles in the order they are walked: tile u (a multiple of BN) holds the positions from
+    // u + (u >= keep_end ? gap : 0) on. Without kept keys that is the position itself, from the window's first
+    // tile on; with them the tiles below keep_end come first and the walk then jumps over the gap.
+    int keep_end = 0, gap = 0, u_first = (first_key / BN) * BN;
+    int low_key = first_key;                             // the earliest key that a row of this tile may read
+    if constexpr (XT) {
+        if (keep_first > 0 && window > 0 && first_key > start) {
+            low_key = start;
+            keep_end = ((min(keep_first, tile_last_pos + 1) + BN - 1) / BN) * BN;
+            if (keep_end >= u_first) {
+                keep_end = 0;                            // the kept keys reach the window: one walk from the start
+            } else {
+                gap = u_first - keep_end;
+            }
+            u_first = (start / BN) * BN;
+        }
+    }
+#define POS_OF(u_) ((u_) + ((u_) >= keep_end ? gap : 0))
 
-    const float scale2 = scale * 1.44269504088896340736f;
+    const float score_scale = XT ? scale * (head_scale != nullptr ? head_scale[head] : 1.f) : 1.f;
+    const float inv_cap = (XT && softcap > 0.f) ? 1.0f / softcap : 0.f;
+    // (with the extras the scores are finished before the maximum is taken; else the scale comes in with the exponent)
+    const float scale2 = (XT ? 1.f : scale) * 1.44269504088896340736f;
     // positions of the first and last row of this wave (wave-uniform, for skipping the mask)
     const int wave_first_pos = pos0 + q_off + wave * QG * 16;
     const int wave_last_pos = wave_first_pos + QG * 16 - 1;
@@ -161,7 +187,7 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
     const int p_shift = (P & (P - 1)) == 0 ? __builtin_ctz(P) : -1;
 #define ROW_OF(kp)                                                                  \
     ([&]() {                                                                        \
-        const int idx_ = min(max((kp), first_key), tile_last_pos) - start;          \
+        const int idx_ = min(max((kp), low_key), tile_last_pos) - start;            \
         const int pi_ = p_shift >= 0 ? (idx_ >> p_shift) : (idx_ / P);              \
         return (pt[pi_] * Hkv + kvh) * P + (idx_ - pi_ * P);                        \
     }())
@@ -185,33 +211,33 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
         }                                                                           \
     }
     // group grp takes the key tiles grp, grp + KSPLIT, grp + 2 KSPLIT, ... counted from c_first
-    const int c_first = (first_key / BN) * BN;
     constexpr int STEP = KSPLIT * BN;                    // from one tile of a group to its next
     int row_next;                                        // row of this thread's key in the tile fetched next
     {
-        const int c_mine = c_first + grp * BN;
-        const int r0 = ROW_OF(c_mine + my_key);
-        row_next = ROW_OF(c_mine + STEP + my_key);
+        const int u_mine = u_first + grp * BN;
+        const int r0 = ROW_OF(POS_OF(u_mine) + my_key);
+        row_next = ROW_OF(POS_OF(u_mine + STEP) + my_key);
         FETCH_ROW(r0)
         STAGE_TO(0)
         FETCH_ROW(row_next)                              // the group's second tile (or a repeat of valid rows if there is none)
-        row_next = ROW_OF(c_mine + 2 * STEP + my_key);
+        row_next = ROW_OF(POS_OF(u_mine + 2 * STEP) + my_key);
     }
     __syncthreads();
 
     int it = 0;
-    for (int c_it = c_first; c_it <= tile_last_pos; c_it += STEP, ++it) {
-        const int c0 = c_it + grp * BN;                  // beyond tile_last_pos: this group sits the pass out
+    for (int u_it = u_first; POS_OF(u_it) <= tile_last_pos; u_it += STEP, ++it) {
+        const int u0 = u_it + grp * BN;
+        const int c0 = POS_OF(u0);                       // beyond tile_last_pos: this group sits the pass out
         const int cur = it & 1;
         const uint16_t* k_cur = K_S(cur);
         const uint16_t* v_cur = V_S(cur);
-        if (c0 + STEP <= tile_last_pos) {
+        if (POS_OF(u0 + STEP) <= tile_last_pos) {
             // the next tile, asked for one pass ago, goes into the other buffer (which every wave left
             // at the last barrier); then the tile after it is asked for
             STAGE_TO(cur ^ 1)
-            if (c0 + 2 * STEP <= tile_last_pos) {
+            if (POS_OF(u0 + 2 * STEP) <= tile_last_pos) {
                 FETCH_ROW(row_next)
-                row_next = ROW_OF(c0 + 3 * STEP + my_key);
+                row_next = ROW_OF(POS_OF(u0 + 3 * STEP) + my_key);
             }
         }
 
@@ -243,8 +269,27 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
         // p = 2^((s - m) * scale * log2(e)) with s the raw score and m the raw maximum of the row: one fused
         // multiply-add and one exponential a score (the scale is positive, so the maximum may be taken first).
         // a tile that lies wholly below every row of the wave and inside every window needs no mask
-        const bool need_mask = (c0 + BN - 1 > wave_first_pos) || (c0 < first_key) ||
-                               (window > 0 && c0 <= wave_last_pos - window);
+        bool need_mask = (c0 + BN - 1 > wave_first_pos) || (c0 < first_key) ||
+                         (window > 0 && c0 <= wave_last_pos - window);
+        if constexpr (XT) {
+            // a tile of kept keys only, below every row of the wave, needs none either
+            if (keep_first > 0 && c0 >= low_key && c0 + BN <= keep_first && c0 + BN - 1 <= wave_first_pos) need_mask = false;
+            // the scores as they enter the softmax: scale and the head's factor, then the soft cap
+#pragma unroll
+            for (int qg = 0; qg < QG; ++qg)
+#pragma unroll
+                for (int st = 0; st < BN / 16; ++st)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        float t = cs[qg][st][i] * score_scale;
+                        if (softcap > 0.f) {
+                            // c tanh(t / c) = c (1 - 2 / (1 + e^(2t/c)))
+                            const float e2 = __builtin_amdgcn_exp2f(t * inv_cap * 2.88539008177792681472f);
+                            t = softcap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e2));
+                        }
+                        cs[qg][st][i] = t;
+                    }
+        }
         uint4_t pw[QG][BN / 32];                         // P as bf16, in the order the B operand wants
 #pragma unroll
         for (int qg = 0; qg < QG; ++qg) {
@@ -256,8 +301,12 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         const int kpos = c0 + st * 16 + 4 * g + i;
-                        bool ok = kpos >= first_key && kpos <= pos_q[qg];
-                        if (window > 0) ok = ok && kpos > pos_q[qg] - window;
+                        bool ok = kpos >= low_key && kpos <= pos_q[qg];
+                        if constexpr (XT) {
+                            if (window > 0) ok = ok && (kpos > pos_q[qg] - window || kpos < keep_first);
+                        } else {
+                            if (window > 0) ok = ok && kpos > pos_q[qg] - window;
+                        }
                         s[st][i] = ok ? cs[qg][st][i] : -INFINITY;
                         mx = fmaxf(mx, s[st][i]);
                     }
@@ -327,6 +376,7 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
 #undef FETCH_ROW
 #undef STAGE_TO
 #undef ROW_OF
+#undef POS_OF
 #undef K_S
 #undef V_S
     MFMA_SETTLE();
@@ -360,12 +410,16 @@ __global__ __launch_bounds__(256 * KSPLIT) __attribute__((amdgpu_waves_per_eu(2)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     acc[qg][dt][i] = acc[qg][dt][i] * a0 + mq[(2 + 4 * dt + i) * 64] * a1;
+            m_run[qg] = m;                               // (the sink's share below is taken against the merged maximum)
         }
     }
     // ---- acc[qg][dt][i] = O^T[d = 16dt + 4g + i][query n of group qg]
 #pragma unroll
     for (int qg = 0; qg < QG; ++qg) {
         if (!q_ok[qg]) continue;
+        if constexpr (XT) {
+            if (sink) l_run[qg] += __builtin_amdgcn_exp2f(-m_run[qg] * scale2);      // the key of score 0 without a value
+        }
         const float inv = l_run[qg] > 0.f ? 1.0f / l_run[qg] : 0.f;
         bf16* op = out + ((size_t)(cu_q[seg] + pos_q[qg] - pos0) * Hq + head) * D;
 #pragma unroll
@@ -385,10 +439,20 @@ extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, int tile_rows, int key_s
                                               const bf16* kp, const bf16* vp, const int* pt,
                                               const int* cup, const int* kvs, const int* cuq,
                                               const int* qs, const int* tiles, int n_tiles, int Hq,
-                                              int Hkv, int P, float scale, int window) {
+                                              int Hkv, int P, float scale, int window, const float* head_scale,
+                                              float softcap, int keep_first, int sink) {
+    const bool extras = head_scale != nullptr || softcap > 0.f || keep_first > 0 || sink != 0;
 #define PRE_LAUNCH(N, QG_, KS_)                                                                    \
-    hipLaunchKernelGGL((attn_prefill_kernel<N, QG_, KS_>), grid, dim3(256 * KS_), 0, st, q, out, kp, vp, pt, \
-                       cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window)
+    do {                                                                                           \
+        if (extras)                                                                                \
+            hipLaunchKernelGGL((attn_prefill_kernel<N, QG_, KS_, true>), grid, dim3(256 * KS_), 0, st, q, out, kp, vp, pt, \
+                               cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window, head_scale, softcap,     \
+                               keep_first, sink);                                                  \
+        else                                                                                       \
+            hipLaunchKernelGGL((attn_prefill_kernel<N, QG_, KS_, false>), grid, dim3(256 * KS_), 0, st, q, out, kp, vp, pt, \
+                               cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window, head_scale, softcap,     \
+                               keep_first, sink);                                                  \
+    } while (0)
 #define PRE_CASE(N)                                                                               \
     case N:                                                                                       \
         if (N <= PRE_WIDE_D16 && tile_rows == 128) {                                              \
@@ -412,7 +476,8 @@ extern "C" int PRE_CAT(ra_pre_part_, PRE_PART)(int D16, int tile_rows, int key_s
 #ifdef PRE_API
 #define PRE_PART_ARGS int D16, int tile_rows, int key_split, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp,    \
     const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs,    \
-    const int* tiles, int n_tiles, int Hq, int Hkv, int P, float scale, int window
+    const int* tiles, int n_tiles, int Hq, int Hkv, int P, float scale, int window, const float* head_scale,   \
+    float softcap, int keep_first, int sink
 extern "C" int ra_pre_part_0(PRE_PART_ARGS);
 extern "C" int ra_pre_part_1(PRE_PART_ARGS);
 extern "C" int ra_pre_part_2(PRE_PART_ARGS);
@@ -430,7 +495,8 @@ extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k
                                          const int* cu_pages, const int* kv_start, const int* cu_q,
                                          const int* q_start, const int* tiles, int n_tiles,
                                          int tile_rows, int key_split, int Hq, int Hkv, int D, int P,
-                                         float scale, int window, void* stream) {
+                                         float scale, int window, const float* head_scale, float softcap,
+                                         int keep_first, int sink, void* stream) {
     if (n_tiles <= 0) return RA_OK;
     if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 ||
         (long long)n_tiles * Hq > 0x7fffffffLL || (tile_rows != ra_attention_prefill_tile_rows(D) && tile_rows != 64))
@@ -447,7 +513,7 @@ extern "C" int ra_attention_prefill_bf16(const void* q, void* out, const void* k
 #define GO(k)                                                                                      \
     rc = ra_pre_part_##k(d16, tile_rows, key_split, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool,           \
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, tiles, \
-                         n_tiles, Hq, Hkv, P, scale, window)
+                         n_tiles, Hq, Hkv, P, scale, window, head_scale, softcap, keep_first, sink)
     switch ((d16 - 1) / 4) {
         case 0: GO(0); break;
         case 1: GO(1); break;

@@ -55,25 +55,27 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     if (q_len <= 0) return;
     const int PS = DPT + DR_PAD;                    // a lane group's rows in LDS, padded against bank conflicts
     const int DP = RS * PS;
+    const int rap = (ra + 3) & ~3, rgp = (rg + 3) & ~3;   // the ranks as rows of whole float4 (zeros beyond)
     float* k_s = smem;                              // [TC][DP]
     float* q_s = k_s + DR_TC * DP;                  // [TC][DP]
     float* g_s = q_s + DR_TC * DP;                  // [TC][DP]
     float* v_s = g_s + DR_TC * DP;                  // [TC][V]
     float* o_s = v_s + DR_TC * V;                   // [TC][V]
-    float* a1_s = o_s + DR_TC * V;                  // [TC][ra]
-    float* g1_s = a1_s + DR_TC * ra;                // [TC][rg]
-    float* beta_s = g1_s + DR_TC * rg;              // [TC]
+    float* a1_s = o_s + DR_TC * V;                  // [TC][rap]
+    float* g1_s = a1_s + DR_TC * rap;               // [TC][rgp]
+    float* beta_s = g1_s + DR_TC * rgp;             // [TC]
+    float* rstd_s = beta_s + DR_TC;                 // [TC]
     // staged: this head's rows of the two low-rank second factors sit in LDS for the whole walk
-    float* wa_s = beta_s + DR_TC;                   // [ra][D]
-    float* wg_s = wa_s + (staged ? ra * D : 0);     // [rg][V]
+    float* wa_s = rstd_s + DR_TC;                   // [rap][D]
+    float* wg_s = wa_s + (staged ? rap * D : 0);    // [rgp][V]
     if (staged) {
-        for (int idx = tid; idx < ra * D; idx += NT) {
+        for (int idx = tid; idx < rap * D; idx += NT) {
             const int r = idx / D, i = idx - r * D;
-            wa_s[idx] = w_a2t[(size_t)r * H * D + h * D + i];
+            wa_s[idx] = r < ra ? w_a2t[(size_t)r * H * D + h * D + i] : 0.f;
         }
-        for (int idx = tid; idx < rg * V; idx += NT) {
+        for (int idx = tid; idx < rgp * V; idx += NT) {
             const int r = idx / V, jj = idx - r * V;
-            wg_s[idx] = w_g2t[(size_t)r * H * V + h * V + jj];
+            wg_s[idx] = r < rg ? w_g2t[(size_t)r * H * V + h * V + jj] : 0.f;
         }
     }
 
@@ -93,13 +95,13 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     for (int c0 = 0; c0 < q_len; c0 += DR_TC) {
         const int nt = min(DR_TC, q_len - c0);
         // ---- what the chunk's rows bring, into LDS
-        for (int idx = tid; idx < nt * ra; idx += NT) {
-            const int tt = idx / ra, r = idx - tt * ra;
-            a1_s[tt * ra + r] = to_f(z[(size_t)(base + c0 + tt) * ld_z + off_a + r]);
+        for (int idx = tid; idx < nt * rap; idx += NT) {
+            const int tt = idx / rap, r = idx - tt * rap;
+            a1_s[idx] = r < ra ? to_f(z[(size_t)(base + c0 + tt) * ld_z + off_a + r]) : 0.f;
         }
-        for (int idx = tid; idx < nt * rg; idx += NT) {
-            const int tt = idx / rg, r = idx - tt * rg;
-            g1_s[tt * rg + r] = to_f(z[(size_t)(base + c0 + tt) * ld_z + off_g + r]);
+        for (int idx = tid; idx < nt * rgp; idx += NT) {
+            const int tt = idx / rgp, r = idx - tt * rgp;
+            g1_s[idx] = r < rg ? to_f(z[(size_t)(base + c0 + tt) * ld_z + off_g + r]) : 0.f;
         }
         if (tid < nt) beta_s[tid] = dr_sigmoid(to_f(z[(size_t)(base + c0 + tid) * ld_z + off_b + h]));
         for (int idx = tid; idx < nt * V; idx += NT) {
@@ -107,25 +109,45 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
             v_s[tt * V + jj] = to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + jj]);
         }
         __syncthreads();
-        for (int idx = tid; idx < nt * Dfull; idx += NT) {
-            const int tt = idx / Dfull, i = idx - tt * Dfull;
-            const int at = tt * DP + (i / DPT) * PS + (i % DPT);
-            float kk = 0.f, qq = 0.f, gg = 1.f;
+        // a thread takes one key channel of four rows at a time: a row of the factor is read once for the four
+        for (int idx = tid; idx < ((nt + 3) >> 2) * Dfull; idx += NT) {
+            const int tg = idx / Dfull, i = idx - tg * Dfull;
+            float a[4] = {0.f, 0.f, 0.f, 0.f};
             if (i < D) {
-                const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
-                qq = to_f(row[kvh * D + i]);
-                kk = to_f(row[G * D + kvh * D + i]);
-                float a = dt_bias[h * D + i];
-                if (staged) {
-                    for (int r = 0; r < ra; ++r) a = fmaf(a1_s[tt * ra + r], wa_s[r * D + i], a);
-                } else {
-                    for (int r = 0; r < ra; ++r) a = fmaf(a1_s[tt * ra + r], w_a2t[(size_t)r * H * D + h * D + i], a);
+                const float* a1 = a1_s + (tg * 4) * rap;          // (rows beyond nt hold older numbers: never used)
+#pragma unroll 2
+                for (int r = 0; r < rap; r += 4) {
+                    float w4[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        w4[x] = staged ? wa_s[(r + x) * D + i]
+                                       : (r + x < ra ? w_a2t[(size_t)(r + x) * H * D + h * D + i] : 0.f);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const float4 c4 = *reinterpret_cast<const float4*>(a1 + k * rap + r);
+                        a[k] = fmaf(c4.x, w4[0], a[k]);
+                        a[k] = fmaf(c4.y, w4[1], a[k]);
+                        a[k] = fmaf(c4.z, w4[2], a[k]);
+                        a[k] = fmaf(c4.w, w4[3], a[k]);
+                    }
                 }
-                gg = expf(neg_a * dr_softplus(a));
             }
-            k_s[at] = kk;
-            q_s[at] = qq;
-            g_s[at] = gg;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int tt = tg * 4 + k;
+                if (tt >= nt) break;
+                const int at = tt * DP + (i / DPT) * PS + (i % DPT);
+                float kk = 0.f, qq = 0.f, gg = 1.f;
+                if (i < D) {
+                    const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
+                    qq = to_f(row[kvh * D + i]);
+                    kk = to_f(row[G * D + kvh * D + i]);
+                    gg = expf(neg_a * dr_softplus(a[k] + dt_bias[h * D + i]));
+                }
+                k_s[at] = kk;
+                q_s[at] = qq;
+                g_s[at] = gg;
+            }
         }
         __syncthreads();
         for (int tt = wave; tt < nt; tt += n_waves) {          // unit vectors: a wave per row
@@ -181,20 +203,42 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
             if (live && rp == 0) o_s[tt * V + j] = o;
         }
         __syncthreads();
-        // ---- norm over the head's read-out, weight, output gate: a wave per row
+        // ---- norm over the head's read-out (a wave per row), then weight and output gate: a thread takes one
+        // column of four rows at a time
         for (int tt = wave; tt < nt; tt += n_waves) {
             float ss = 0.f;
             for (int jj = lane; jj < V; jj += 64) ss = fmaf(o_s[tt * V + jj], o_s[tt * V + jj], ss);
-            const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
-            for (int jj = lane; jj < V; jj += 64) {
-                float gate = 0.f;
-                if (staged) {
-                    for (int r = 0; r < rg; ++r) gate = fmaf(g1_s[tt * rg + r], wg_s[r * V + jj], gate);
-                } else {
-                    for (int r = 0; r < rg; ++r) gate = fmaf(g1_s[tt * rg + r], w_g2t[(size_t)r * H * V + h * V + jj], gate);
+            ss = wave_sum(ss);
+            if (lane == 0) rstd_s[tt] = 1.0f / sqrtf(ss / (float)V + eps);
+        }
+        __syncthreads();
+        for (int idx = tid; idx < ((nt + 3) >> 2) * V; idx += NT) {
+            const int tg = idx / V, jj = idx - tg * V;
+            float gt[4] = {0.f, 0.f, 0.f, 0.f};
+            const float* g1 = g1_s + (tg * 4) * rgp;
+#pragma unroll 2
+            for (int r = 0; r < rgp; r += 4) {
+                float w4[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    w4[x] = staged ? wg_s[(r + x) * V + jj]
+                                   : (r + x < rg ? w_g2t[(size_t)(r + x) * H * V + h * V + jj] : 0.f);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const float4 c4 = *reinterpret_cast<const float4*>(g1 + k * rgp + r);
+                    gt[k] = fmaf(c4.x, w4[0], gt[k]);
+                    gt[k] = fmaf(c4.y, w4[1], gt[k]);
+                    gt[k] = fmaf(c4.z, w4[2], gt[k]);
+                    gt[k] = fmaf(c4.w, w4[3], gt[k]);
                 }
+            }
+            const float nw = norm_w[jj];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int tt = tg * 4 + k;
+                if (tt >= nt) break;
                 out[(size_t)(base + c0 + tt) * H * V + h * V + jj] =
-                    from_f<T>(o_s[tt * V + jj] * rstd * norm_w[jj] * dr_sigmoid(gate));
+                    from_f<T>(o_s[tt * V + jj] * rstd_s[tt] * nw * dr_sigmoid(gt[k]));
             }
         }
         __syncthreads();
@@ -207,10 +251,13 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
 }
 
 static size_t delta_rule_lds(int DPT, int RS, int V, int ra, int rg) {
-    return sizeof(float) * ((size_t)DR_TC * (3 * RS * (DPT + DR_PAD) + 2 * V + ra + rg) + DR_TC);
+    const int rap = (ra + 3) & ~3, rgp = (rg + 3) & ~3;
+    return sizeof(float) * ((size_t)DR_TC * (3 * RS * (DPT + DR_PAD) + 2 * V + rap + rgp) + 2 * DR_TC);
 }
 // the low-rank factors' rows of one head beside that, if they fit
-static size_t delta_rule_staged(int D, int V, int ra, int rg) { return sizeof(float) * ((size_t)ra * D + (size_t)rg * V); }
+static size_t delta_rule_staged(int D, int V, int ra, int rg) {
+    return sizeof(float) * ((size_t)((ra + 3) & ~3) * D + (size_t)((rg + 3) & ~3) * V);
+}
 #define DR_LDS_LIMIT (156 * 1024)
 
 // The split of a column's rows over lanes: RS lanes (a power of two) of DPT rows each.

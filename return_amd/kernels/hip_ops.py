@@ -82,7 +82,7 @@ def _declare(lib):
         "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, I, P],
         "ra_attention_decode_static_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_merge_waves": [I],
-        "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P],
+        "ra_attention_prefill_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, F, I, I, P],
         "ra_attention_prefill_tile_rows": [I],
         "ra_sample": [P, I, I, P, P, P, P, P, P],
         "ra_sample_traced": [P, I, I, P, P, P, P, P, P, P],
@@ -987,9 +987,24 @@ class HipOps:
             split = self.prefill_key_split or small_split or self._prefill_key_split(step, rows, tiles.shape[0] * n_q)
             self._check(self.lib.ra_attention_prefill_bf16(
                 _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], rows,
-                split, n_q, n_kv, D, P, float(scale), window, self._stream()),
-                "attention_prefill_bf16")
+                split, n_q, n_kv, D, P, float(scale), window, _ptr(head_scale), softcap, keep_first,
+                1 if sink else 0, self._stream()), "attention_prefill_bf16")
 
+        def plain_part(toks, n_tok):
+            self._check(self.lib.ra_attention_plain(
+                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
+                n_q, n_kv, D, P, float(scale), window, _code(q.dtype), _ptr(head_scale), softcap, keep_first,
+                1 if sink else 0, self._stream()), "attention_plain")
+
+        if plain_only and q.dtype == torch.bfloat16 and D % 16 == 0 and D <= 256 and bool(step.prefill_tiles) \
+                and step.n_prefill_tokens > 0:
+            # the prompts' kernel takes the extras, the single tokens' kernel does not: the requests that bring
+            # one token go to the plain kernel through the list of their rows
+            prefill_part()
+            if step.n_decode > 0:
+                rows = step.cu_q.index_select(0, step.decode_segs.to(torch.int64)).contiguous()
+                plain_part(rows, step.n_decode)
+            return
         if fast_decode and fast_prefill and step.n_prefill_tokens > 0:
             # A step of prompt portions beside decoded tokens: the two kernels work on different rows of q and
             # out, one is bound by memory and the other by the matrix cores and the latency inside its waves,
@@ -1019,10 +1034,7 @@ class HipOps:
         if fast_prefill:
             prefill_part()
             return
-        self._check(self.lib.ra_attention_plain(
-            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(toks), step.n_seqs, n_tok,
-            n_q, n_kv, D, P, float(scale), window, _code(q.dtype), _ptr(head_scale), softcap, keep_first,
-            1 if sink else 0, self._stream()), "attention_plain")
+        plain_part(toks, n_tok)
 
     def _decode_splits(self, step, n_q, n_kv, D, window):
         """Keys per split of the decode attention, the most splits a request has, and whether a
