@@ -49,8 +49,10 @@ struct DecodeRange {
     int n_splits;             // splits that hold keys for this request
 };
 
+// keep_first > 0: the keys at positions below it stay readable whatever the window; where the window has
+// moved past them they are one more split, the request's last.
 __device__ __forceinline__ DecodeRange decode_range(int pos_q, int start, int window,
-                                                    int split_tokens, int sp) {
+                                                    int split_tokens, int sp, int keep_first = 0) {
     int first = start;
     if (window > 0 && pos_q - window + 1 > first) first = pos_q - window + 1;
     const int split0 = first / split_tokens;
@@ -59,8 +61,25 @@ __device__ __forceinline__ DecodeRange decode_range(int pos_q, int start, int wi
     r.lo = max(first, s_abs * split_tokens);
     r.hi = min(pos_q, (s_abs + 1) * split_tokens - 1);
     r.n_splits = pos_q / split_tokens - split0 + 1;
+    if (keep_first > 0 && first > start) {
+        if (sp == r.n_splits) {
+            r.lo = start;
+            r.hi = min(keep_first, first) - 1;
+        }
+        r.n_splits += 1;
+    }
     return r;
 }
+
+// The optional extras (XT): head_scale[h] multiplies the scale of query head h; softcap c turns a score s
+// into c tanh(s / c); keep_first as above; sink adds one to the softmax's denominator (a key of score 0
+// that has no value), where the splits are merged.
+struct DecodeExtras {
+    const float* head_scale;
+    float softcap;
+    int keep_first;
+    int sink;
+};
 
 // What the kernel needs to prepare the new token's q, k and v itself (the work of the q/k/v
 // preparation kernel: per-head RMSNorm of q and k, rotation, k and v into the cache;
@@ -200,7 +219,7 @@ __host__ __device__ constexpr int dec_region_bytes(int D) {
 // per (request, kv head), wave w takes split w, and the waves' sums are merged through LDS here
 // (the same sums in the same order as the merge kernel), so that nothing goes through memory and
 // no second kernel runs; for requests whose splits fit one workgroup.
-template <int D16, bool FUSED>
+template <int D16, bool FUSED, bool XT>
 __global__ __launch_bounds__(D16 <= 8 ? 512 : 256) __attribute__((amdgpu_waves_per_eu(D16 <= 8 ? 2 : 1)))
 void attn_decode_kernel(
     const bf16* __restrict__ q, float* __restrict__ part_acc, float* __restrict__ part_ml,
@@ -209,7 +228,7 @@ void attn_decode_kernel(
     const int* __restrict__ kv_start, const int* __restrict__ cu_q,
     const int* __restrict__ q_start, const int* __restrict__ seg_ids, int Hq, int Hkv, int P,
     float scale, int window, int split_tokens, int max_splits, DecodeFused fz, int merge_waves,
-    bf16* __restrict__ out) {
+    bf16* __restrict__ out, DecodeExtras ex) {
     constexpr int D = 16 * D16;
     constexpr int D32 = D / 32;                 // full MFMA x32 steps
     constexpr bool TAIL16 = (D % 32) != 0;      // one more step, upper k half zero
@@ -241,7 +260,7 @@ void attn_decode_kernel(
     // A merging workgroup cuts its own request into merge_waves even splits (counted from
     // position 0), whatever the longest request of the step is.
     if (merge_waves > 1) split_tokens = max(1, (pos_q + DEC_CHUNK * merge_waves) / (DEC_CHUNK * merge_waves)) * DEC_CHUNK;
-    const DecodeRange rg = decode_range(pos_q, start, window, split_tokens, sp);
+    const DecodeRange rg = decode_range(pos_q, start, window, split_tokens, sp, XT ? ex.keep_first : 0);
     const bool empty = rg.lo > rg.hi;            // a split beyond the request's keys
     if (empty && merge_waves == 1) return;       // (in a merging workgroup the wave stays for the barrier, with no keys)
     const int* pt = page_table + first_page;
@@ -356,6 +375,10 @@ void attn_decode_kernel(
     }
 
     const float scale2 = scale * 1.44269504088896340736f;      // scores in the base-2 domain
+    // XT: this lane's head has a factor of its own on the scale, and the score is capped before it enters the softmax
+    [[maybe_unused]] const float head_scale =
+        XT ? scale * ((ex.head_scale != nullptr && n < G) ? ex.head_scale[h0 + n] : 1.f) : 0.f;
+    [[maybe_unused]] const float inv_cap = (XT && ex.softcap > 0.f) ? 1.0f / ex.softcap : 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     float4_t acc[D16];                           // acc[dt][i] = O^T[d = 16dt + 4g + i][head n]
 #pragma unroll
@@ -406,7 +429,16 @@ void attn_decode_kernel(
             for (int i = 0; i < 4; ++i) {
                 const int kp_abs = c0 + st * 16 + 4 * g + i;
                 const bool ok = kp_abs >= rg.lo && kp_abs <= key_hi;
-                s[st][i] = ok ? cs[st][i] * scale2 : -INFINITY;
+                if constexpr (XT) {
+                    float t = cs[st][i] * head_scale;
+                    if (ex.softcap > 0.f) {                 // c tanh(t / c) = c (1 - 2 / (1 + e^(2t/c)))
+                        const float e2 = __builtin_amdgcn_exp2f(t * inv_cap * 2.88539008177792681472f);
+                        t = ex.softcap * (1.f - 2.f * __builtin_amdgcn_rcpf(1.f + e2));
+                    }
+                    s[st][i] = ok ? t * 1.44269504088896340736f : -INFINITY;
+                } else {
+                    s[st][i] = ok ? cs[st][i] * scale2 : -INFINITY;
+                }
                 mx = fmaxf(mx, s[st][i]);
             }
         }
@@ -518,6 +550,9 @@ void attn_decode_kernel(
                 o[2] = fmaf(a[2], e, o[2]); o[3] = fmaf(a[3], e, o[3]);
                 l += other[16 * D + 2 * hn + 1] * e;
             }
+            if constexpr (XT) {
+                if (ex.sink) l += __builtin_amdgcn_exp2f(-mx);       // the key of score 0 without a value
+            }
             const float inv = l > 0.f ? 1.0f / l : 0.f;
             const uint2 packed = {pack2(o[0] * inv, o[1] * inv), pack2(o[2] * inv, o[3] * inv)};
             *reinterpret_cast<uint2*>(out + ((size_t)t * Hq + h0 + hn) * D + 4 * d4) = packed;
@@ -541,14 +576,15 @@ void attn_decode_kernel(
 #define DEC_CAT2(a, b) a##b
 #define DEC_CAT(a, b) DEC_CAT2(a, b)
 // head sizes 16*(4*DEC_PART+1) .. 16*(4*DEC_PART+4)
-template <int N, bool FUSED>
+template <int N, bool FUSED, bool XT>
 static int dec_launch_one(dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm, const bf16* kp,
                           const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq,
                           const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,
-                          int split_tokens, int max_splits, DecodeFused fz, int merge_waves, bf16* out) {
+                          int split_tokens, int max_splits, DecodeFused fz, int merge_waves, bf16* out,
+                          DecodeExtras ex) {
     constexpr int D = 16 * N;
     const size_t lds = (size_t)merge_waves * (dec_region_bytes(D) + (FUSED ? 4 * D : 0));
-    auto kern = attn_decode_kernel<N, FUSED>;
+    auto kern = attn_decode_kernel<N, FUSED, XT>;
     static size_t allowed = 64 * 1024;                        // per instantiation: raised when needed
     if (lds > allowed) {
         if (lds > 160 * 1024 ||
@@ -558,7 +594,7 @@ static int dec_launch_one(dim3 grid, hipStream_t st, const bf16* q, float* pa, f
         allowed = lds;
     }
     hipLaunchKernelGGL(kern, grid, dim3(64 * merge_waves), lds, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs,
-                       segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz, merge_waves, out);
+                       segs, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz, merge_waves, out, ex);
     return RA_OK;
 }
 
@@ -567,20 +603,26 @@ extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t s
                                               const int* cup, const int* kvs, const int* cuq,
                                               const int* qs, const int* segs, int Hq, int Hkv, int P,
                                               float scale, int window, int split_tokens,
-                                              int max_splits, DecodeFused fz, int merge_waves, bf16* out) {
+                                              int max_splits, DecodeFused fz, int merge_waves, bf16* out,
+                                              DecodeExtras ex) {
 #define DEC_ARGS grid, st, q, pa, pm, kp, vp, pt, cup, kvs, cuq, qs, segs, Hq, Hkv, P, scale, window, \
-                 split_tokens, max_splits, fz, merge_waves, out
+                 split_tokens, max_splits, fz, merge_waves, out, ex
+    const bool extras = ex.head_scale != nullptr || ex.softcap > 0.f || ex.keep_first > 0 || ex.sink != 0;
     if (fz.qkv != nullptr) {                      // head sizes 64, 128, 192, 256: one of them in each part
-        if (D16 != 4 * DEC_PART + 4) return RA_ERR_ARG;
-        return dec_launch_one<4 * DEC_PART + 4, true>(DEC_ARGS);
+        if (D16 != 4 * DEC_PART + 4 || extras) return RA_ERR_ARG;
+        return dec_launch_one<4 * DEC_PART + 4, true, false>(DEC_ARGS);
     }
+#define DEC_CASE(N_)                                                                  \
+    case N_:                                                                          \
+        return extras ? dec_launch_one<N_, false, true>(DEC_ARGS) : dec_launch_one<N_, false, false>(DEC_ARGS);
     switch (D16) {
-        case 4 * DEC_PART + 1: return dec_launch_one<4 * DEC_PART + 1, false>(DEC_ARGS);
-        case 4 * DEC_PART + 2: return dec_launch_one<4 * DEC_PART + 2, false>(DEC_ARGS);
-        case 4 * DEC_PART + 3: return dec_launch_one<4 * DEC_PART + 3, false>(DEC_ARGS);
-        case 4 * DEC_PART + 4: return dec_launch_one<4 * DEC_PART + 4, false>(DEC_ARGS);
+        DEC_CASE(4 * DEC_PART + 1)
+        DEC_CASE(4 * DEC_PART + 2)
+        DEC_CASE(4 * DEC_PART + 3)
+        DEC_CASE(4 * DEC_PART + 4)
         default: return RA_ERR_ARG;
     }
+#undef DEC_CASE
 #undef DEC_ARGS
 }
 #endif  // DEC_PART
@@ -590,7 +632,7 @@ extern "C" int DEC_CAT(ra_dec_part_, DEC_PART)(int D16, dim3 grid, hipStream_t s
 #define DEC_PART_ARGS int D16, dim3 grid, hipStream_t st, const bf16* q, float* pa, float* pm,        \
     const bf16* kp, const bf16* vp, const int* pt, const int* cup, const int* kvs, const int* cuq,   \
     const int* qs, const int* segs, int Hq, int Hkv, int P, float scale, int window,                 \
-    int split_tokens, int max_splits, DecodeFused fz, int merge_waves, bf16* out
+    int split_tokens, int max_splits, DecodeFused fz, int merge_waves, bf16* out, DecodeExtras ex
 extern "C" int ra_dec_part_0(DEC_PART_ARGS);
 extern "C" int ra_dec_part_1(DEC_PART_ARGS);
 extern "C" int ra_dec_part_2(DEC_PART_ARGS);
@@ -615,7 +657,8 @@ template <int GROUPS>
 __global__ __launch_bounds__(128 * GROUPS) void attn_decode_combine_kernel(
     const float* __restrict__ part_acc, const float* __restrict__ part_ml, bf16* __restrict__ out,
     const int* __restrict__ kv_start, const int* __restrict__ cu_q, const int* __restrict__ q_start,
-    const int* __restrict__ seg_ids, int Hq, int D, int window, int split_tokens, int max_splits) {
+    const int* __restrict__ seg_ids, int Hq, int D, int window, int split_tokens, int max_splits,
+    int keep_first, int sink) {
     const int di = blockIdx.x, head = blockIdx.y, tid = threadIdx.x & 127, grp = threadIdx.x >> 7;
     // this group's run of splits: [first, first + per)
     const int per = GROUPS == 1 ? max_splits : (max_splits + GROUPS - 1) / GROUPS;
@@ -638,7 +681,7 @@ __global__ __launch_bounds__(128 * GROUPS) void attn_decode_combine_kernel(
     }
     const int seg = seg_ids ? seg_ids[di] : di;
     const int t = cu_q ? cu_q[seg] : seg;
-    const DecodeRange rg = decode_range(q_start[seg], kv_start[seg], window, split_tokens, 0);
+    const DecodeRange rg = decode_range(q_start[seg], kv_start[seg], window, split_tokens, 0, keep_first);
     const int ns_all = min(rg.n_splits, max_splits);
     const int ns = max(0, min(ns_all - first, per));        // splits of this group that hold keys
     float m = -INFINITY;                                   // (the maxima are base-2 exponents)
@@ -681,7 +724,9 @@ __global__ __launch_bounds__(128 * GROUPS) void attn_decode_combine_kernel(
             o0 = fmaf(v[2], w, o0);
             o1 = fmaf(v[3], w, o1);
         }
+        m = mx;
     }
+    if (sink) l += __builtin_amdgcn_exp2f(-m);             // the key of score 0 without a value (base-2 exponents)
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     bf16* o = out + ((size_t)t * Hq + head) * D;
     if (tid < D) o[tid] = from_f<bf16>(o0 * inv);
@@ -707,7 +752,7 @@ static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const 
                          const int* page_table, const int* cu_pages, const int* kv_start, const int* cu_q,
                          const int* q_start, const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
                          float scale, int window, int split_tokens, int max_splits, DecodeFused fz,
-                         int merge, hipStream_t st) {
+                         int merge, hipStream_t st, DecodeExtras ex = DecodeExtras{nullptr, 0.f, 0, 0}) {
     if (n_dec <= 0) return RA_OK;
     if (D % 16 != 0 || D < 16 || D > 256 || Hkv <= 0 || Hq % Hkv != 0 ||
         split_tokens <= 0 || split_tokens % DEC_CHUNK != 0 || max_splits <= 0 || max_splits > 65535 || P <= 0)
@@ -721,7 +766,7 @@ static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const 
     const int d16 = D / 16;
 #define DEC_GO(N) rc = ra_dec_part_##N(d16, grid, st, qq, pa, pm, kp, vp, page_table, cu_pages, kv_start, cu_q, \
                                        q_start, seg_ids, Hq, Hkv, P, scale, window, split_tokens, max_splits, fz, \
-                                       merge_waves, (bf16*)out)
+                                       merge_waves, (bf16*)out, ex)
     switch ((d16 - 1) / 4) {
         case 0: DEC_GO(0); break;
         case 1: DEC_GO(1); break;
@@ -734,7 +779,8 @@ static int decode_launch(const bf16* qq, void* out, float* pa, float* pm, const 
     if (hipGetLastError() != hipSuccess) return RA_ERR_LAUNCH;
     if (merge) return RA_OK;
 #define DEC_COMBINE(G) hipLaunchKernelGGL(attn_decode_combine_kernel<G>, dim3(n_dec, Hq), dim3(128 * G), 0, st, pa, pm, \
-                                          (bf16*)out, kv_start, cu_q, q_start, seg_ids, Hq, D, window, split_tokens, max_splits)
+                                          (bf16*)out, kv_start, cu_q, q_start, seg_ids, Hq, D, window, split_tokens, max_splits, \
+                                          ex.keep_first, ex.sink)
     const int groups = (max_splits + COMBINE_AHEAD - 1) / COMBINE_AHEAD;
     if (groups <= 1) DEC_COMBINE(1);
     else if (groups <= 2) DEC_COMBINE(2);
@@ -755,6 +801,24 @@ extern "C" int ra_attention_decode_bf16(const void* q, void* out, void* part_acc
     return decode_launch((const bf16*)q, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
                          (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
                          Hkv, D, P, scale, window, split_tokens, max_splits, none, merge, (hipStream_t)stream);
+}
+
+// The same with the optional extras: head_scale (fp32 [Hq] or null), softcap (0: none), keep_first (the
+// keys below it are one more split where the window has moved past them: max_splits counts it), sink.
+extern "C" int ra_attention_decode_extras_bf16(const void* q, void* out, void* part_acc, void* part_ml,
+                                               const void* k_pool, const void* v_pool,
+                                               const int* page_table, const int* cu_pages,
+                                               const int* kv_start, const int* cu_q, const int* q_start,
+                                               const int* seg_ids, int n_dec, int Hq, int Hkv, int D, int P,
+                                               float scale, int window, int split_tokens, int max_splits,
+                                               int merge, const float* head_scale, float softcap, int keep_first,
+                                               int sink, void* stream) {
+    DecodeFused none = {};
+    if (softcap < 0.f || keep_first < 0) return RA_ERR_ARG;
+    const DecodeExtras ex = {head_scale, softcap, window > 0 ? keep_first : 0, sink};
+    return decode_launch((const bf16*)q, out, (float*)part_acc, (float*)part_ml, (const bf16*)k_pool,
+                         (const bf16*)v_pool, page_table, cu_pages, kv_start, cu_q, q_start, seg_ids, n_dec, Hq,
+                         Hkv, D, P, scale, window, split_tokens, max_splits, none, merge, (hipStream_t)stream, ex);
 }
 
 // The same for requests whose new token has not been prepared: qkv [tokens, (Hq + 2 Hkv) D] as the

@@ -79,6 +79,7 @@ def _declare(lib):
         "ra_add_bias": [P, P, L, I, I, P],
         "ra_qk_prepare": [P, I, I, I, I, P, P, P, P, I, P, P, P, P, I, L, I, P],
         "ra_attention_decode_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
+        "ra_attention_decode_extras_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P, F, I, I, P],
         "ra_attention_decode_fused_bf16": [P, P, P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, P, P, F, P, P, I, P],
         "ra_attention_decode_static_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, F, I, I, I, I, P],
         "ra_attention_decode_merge_waves": [I],
@@ -953,18 +954,27 @@ class HipOps:
             self._want(head_scale, "head scale", torch.float32, 1)
             if head_scale.shape[0] != n_q:
                 raise KernelError(f"attention: head scale {tuple(head_scale.shape)} for {n_q} heads")
-        plain_only = head_scale is not None or softcap > 0.0 or keep_first > 0 or sink
-        fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256 and not plain_only
+        extras = head_scale is not None or softcap > 0.0 or keep_first > 0 or sink
+        fast_decode = q.dtype == torch.bfloat16 and step.n_decode > 0 and D % 16 == 0 and D <= 256
         fast_prefill = q.dtype == torch.bfloat16 and bool(step.prefill_tiles) and D % 16 == 0 and D <= 256 and \
-            (fast_decode or step.n_decode == 0) and not plain_only
+            (fast_decode or step.n_decode == 0)
 
         def decode_part():
             S, max_splits, merge = self._decode_splits(step, n_q, n_kv, D, window)
+            if keep_first > 0 and window > 0:
+                max_splits += 1                  # the kept keys below the window are a split of their own
             nd = step.n_decode
             part_acc = part_ml = None
             if not merge:
                 part_acc = torch.empty(nd, n_q, max_splits, D, dtype=torch.float32, device=self.device)
                 part_ml = torch.empty(nd, n_q, max_splits, 2, dtype=torch.float32, device=self.device)
+            if extras:
+                self._check(self.lib.ra_attention_decode_extras_bf16(
+                    _ptr(q), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(k_pool), _ptr(v_pool), *tabs,
+                    _ptr(step.decode_segs), nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
+                    1 if merge else 0, _ptr(head_scale), softcap, keep_first, 1 if sink else 0, self._stream()),
+                    "attention_decode_extras_bf16")
+                return
             self._check(self.lib.ra_attention_decode_bf16(
                 _ptr(q), _ptr(out), _ptr(part_acc), _ptr(part_ml), _ptr(k_pool), _ptr(v_pool), *tabs,
                 _ptr(step.decode_segs), nd, n_q, n_kv, D, P, float(scale), window, S, max_splits,
@@ -996,15 +1006,6 @@ class HipOps:
                 n_q, n_kv, D, P, float(scale), window, _code(q.dtype), _ptr(head_scale), softcap, keep_first,
                 1 if sink else 0, self._stream()), "attention_plain")
 
-        if plain_only and q.dtype == torch.bfloat16 and D % 16 == 0 and D <= 256 and bool(step.prefill_tiles) \
-                and step.n_prefill_tokens > 0:
-            # the prompts' kernel takes the extras, the single tokens' kernel does not: the requests that bring
-            # one token go to the plain kernel through the list of their rows
-            prefill_part()
-            if step.n_decode > 0:
-                rows = step.cu_q.index_select(0, step.decode_segs.to(torch.int64)).contiguous()
-                plain_part(rows, step.n_decode)
-            return
         if fast_decode and fast_prefill and step.n_prefill_tokens > 0:
             # A step of prompt portions beside decoded tokens: the two kernels work on different rows of q and
             # out, one is bound by memory and the other by the matrix cores and the latency inside its waves,

@@ -164,12 +164,18 @@ ATTN = [  # Hq, Hkv, D, P, [(q_len, q_start)], window, keep_first, softcap
     (2, 1, 128, 16, [(130, 200)], 70, 3, 50.0),
     (5, 5, 48, 32, [(1, 1000), (3, 997)], 64, 64, 2.0),
     (8, 2, 20, 4, [(1, 77), (19, 58)], 5, 1, 0.0),
+    (4, 2, 64, 16, [(1, 300), (1, 90), (1, 2000)], 0, 0, 10.0),       # no window: a request's splits may be merged in one workgroup
+    (16, 2, 128, 16, [(1, 700), (1, 64), (1, 1), (1, 5000)], 1024, 64, 30.0),
+    (16, 2, 128, 16, [(1, 1500), (300, 1200), (1, 8)], 128, 64, 30.0),
 ]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("Hq,Hkv,D,P,segs,window,keep,cap", ATTN)
-def test_attention_with_kept_keys_cap_temperature_and_sink(ops, ref, dtype, Hq, Hkv, D, P, segs, window, keep, cap):
+def test_attention_with_kept_keys_cap_temperature_and_sink(ops, ref, dtype, Hq, Hkv, D, P, segs, window, keep, cap,
+                                                           monkeypatch):
+    if window == 0:
+        monkeypatch.setattr(ops, "decode_merge_round", 1)         # (the merge inside the workgroup, where it applies)
     q_lens, q_starts = [s[0] for s in segs], [s[1] for s in segs]
     need = [-(-(a + b) // P) for a, b in segs]
     perm = torch.randperm(sum(need) + 3, generator=torch.Generator().manual_seed(5)).tolist()
