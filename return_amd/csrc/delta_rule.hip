@@ -1,28 +1,27 @@
-// Gated delta rule with one decay per key channel, as one kernel over the rows of a step.
+// Gated delta rule with one decay per key channel, over the rows of a step.
 //
 // Per head, with S [D, V] in 32-bit carried from token to token for each request:
 //     S <- diag(g_t) S;   u = beta_t (v_t - S^T k_t);   S <- S + k_t u^T;   o_t = S^T q_t
 // (the read-out sees the token's own write). Around it, all in 32-bit:
 //     q_t, k_t: unit vectors per head, x / sqrt(sum x^2 + 1e-6), q times D^-1/2
 //     beta_t = sigmoid(b_t)
-//     g_t[i] = exp(-exp(A_log[h]) * softplus(dt_bias[h,i] + sum_r a1_t[r] * Wa2[h,i,r]))
-//     out_t[j] = o_t[j] / sqrt(mean_j o_t[j]^2 + eps) * norm_w[j] * sigmoid(sum_r g1_t[r] * Wg2[h,j,r])
+//     g_t[i] = exp(-exp(A_log[h]) * softplus(a_t[h,i] + dt_bias[h,i]))
+//     out_t[j] = o_t[j] / sqrt(mean_j o_t[j]^2 + eps) * norm_w[j] * sigmoid(c_t[h,j])
 // Inputs: qkv, the rows after the short convolution and its activation, [q heads | k heads | v heads]
-// (G heads of D for q and k, H heads of V for v; head h reads q/k head h / (H/G)); z, the rows of the
-// fused input projection, of which beta (H columns at off_b), a1 (ra columns at off_a) and g1 (rg
-// columns at off_g) are read; the second factors of the two low-rank maps transposed, fp32
-// [ra, H*D] and [rg, H*V].
+// (G heads of D for q and k, H heads of V for v; head h reads q/k head h / (H/G)); b, one column per
+// head of some wider rows; ag, rows [a: H*D | c: H*V], the decay's and the output gate's projections.
 //
-// A workgroup takes one (head, request) and walks the request's rows in chunks of DR_TC: first
-// everything that does not depend on S is prepared for the chunk in LDS by all threads (the decay's
-// low-rank map, whose second factor's rows for this head are copied into LDS once when they fit,
-// softplus, exponentials, the unit vectors), then the recurrence runs over the chunk
-// without a barrier, then the chunk's read-outs are normed, gated and stored. In the recurrence a
-// column j of S belongs to RS neighbouring lanes, each with DPT rows in registers; the two sums
-// over rows are finished by lane swaps.
+// Two kernels. The recurrence: a workgroup takes (head, VB columns of S, request) and walks the
+// request's rows in chunks of DR_TC; for a chunk everything that does not depend on S (decays, unit
+// vectors, beta) is prepared in LDS by all threads, then the recurrence runs over the chunk without a
+// barrier and writes the read-outs o in 32-bit. A column j of S belongs to RS neighbouring lanes, each
+// with DPT rows in registers; the two sums over rows are finished by data-parallel moves. Columns of
+// one head are independent, so a head is spread over V / VB workgroups: the walk over the tokens is the
+// long pole, and it is as long for 16 columns as for 128. The output kernel norms a head's read-out
+// over all its columns, weighs and gates it: a wave per (row, head).
 #include "common.h"
 
-#define DR_TC 16
+#define DR_TC 32
 #define DR_PAD 4
 
 __device__ __forceinline__ float dr_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
@@ -42,45 +41,28 @@ __device__ __forceinline__ float dr_group_sum(float v, int RS) {
 }
 
 template <typename T, int DPT>
-__global__ __launch_bounds__(512) void delta_rule_kernel(
-    const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ z, long long ld_z, int off_b, int off_a,
-    int ra, int off_g, int rg, const float* __restrict__ w_a2t, const float* __restrict__ w_g2t,
-    const float* __restrict__ A_log, const float* __restrict__ dt_bias, const float* __restrict__ norm_w,
-    float eps, float* __restrict__ S, const int* __restrict__ cu_q, const int* __restrict__ slot_ids,
-    T* __restrict__ out, int H, int G, int D, int V, int RS, int staged) {
+__global__ __launch_bounds__(256) void delta_rule_kernel(
+    const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ b, long long ld_b, const T* __restrict__ ag,
+    long long ld_ag, const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ S,
+    const int* __restrict__ cu_q, const int* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int D, int V,
+    int RS, int VB) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int tid = threadIdx.x, NT = blockDim.x, lane = tid & 63, wave = tid >> 6, n_waves = NT >> 6;
-    const int h = blockIdx.x, s = blockIdx.y, kvh = h / (H / G);
+    const int col_blocks = (V + VB - 1) / VB;
+    const int h = blockIdx.x / col_blocks, j0 = (blockIdx.x - h * col_blocks) * VB;
+    const int s = blockIdx.y, kvh = h / (H / G);
     const int base = cu_q[s], q_len = cu_q[s + 1] - base;
     if (q_len <= 0) return;
     const int PS = DPT + DR_PAD;                    // a lane group's rows in LDS, padded against bank conflicts
     const int DP = RS * PS;
-    const int rap = (ra + 3) & ~3, rgp = (rg + 3) & ~3;   // the ranks as rows of whole float4 (zeros beyond)
     float* k_s = smem;                              // [TC][DP]
     float* q_s = k_s + DR_TC * DP;                  // [TC][DP]
     float* g_s = q_s + DR_TC * DP;                  // [TC][DP]
-    float* v_s = g_s + DR_TC * DP;                  // [TC][V]
-    float* o_s = v_s + DR_TC * V;                   // [TC][V]
-    float* a1_s = o_s + DR_TC * V;                  // [TC][rap]
-    float* g1_s = a1_s + DR_TC * rap;               // [TC][rgp]
-    float* beta_s = g1_s + DR_TC * rgp;             // [TC]
-    float* rstd_s = beta_s + DR_TC;                 // [TC]
-    // staged: this head's rows of the two low-rank second factors sit in LDS for the whole walk
-    float* wa_s = rstd_s + DR_TC;                   // [rap][D]
-    float* wg_s = wa_s + (staged ? rap * D : 0);    // [rgp][V]
-    if (staged) {
-        for (int idx = tid; idx < rap * D; idx += NT) {
-            const int r = idx / D, i = idx - r * D;
-            wa_s[idx] = r < ra ? w_a2t[(size_t)r * H * D + h * D + i] : 0.f;
-        }
-        for (int idx = tid; idx < rgp * V; idx += NT) {
-            const int r = idx / V, jj = idx - r * V;
-            wg_s[idx] = r < rg ? w_g2t[(size_t)r * H * V + h * V + jj] : 0.f;
-        }
-    }
+    float* v_s = g_s + DR_TC * DP;                  // [TC][VB]
+    float* beta_s = v_s + DR_TC * VB;               // [TC]
 
-    const int j = tid / RS, rp = tid % RS;
-    const bool live = j < V;
+    const int jl = tid / RS, rp = tid % RS, j = j0 + jl;
+    const bool live = jl < VB && j < V;
     float* Sh = S + ((size_t)slot_ids[s] * H + h) * D * V;
     float st[DPT];
 #pragma unroll
@@ -95,59 +77,25 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     for (int c0 = 0; c0 < q_len; c0 += DR_TC) {
         const int nt = min(DR_TC, q_len - c0);
         // ---- what the chunk's rows bring, into LDS
-        for (int idx = tid; idx < nt * rap; idx += NT) {
-            const int tt = idx / rap, r = idx - tt * rap;
-            a1_s[idx] = r < ra ? to_f(z[(size_t)(base + c0 + tt) * ld_z + off_a + r]) : 0.f;
+        if (tid < nt) beta_s[tid] = dr_sigmoid(to_f(b[(size_t)(base + c0 + tid) * ld_b + h]));
+        for (int idx = tid; idx < nt * VB; idx += NT) {
+            const int tt = idx / VB, jj = idx - tt * VB;
+            v_s[idx] = j0 + jj < V ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
         }
-        for (int idx = tid; idx < nt * rgp; idx += NT) {
-            const int tt = idx / rgp, r = idx - tt * rgp;
-            g1_s[idx] = r < rg ? to_f(z[(size_t)(base + c0 + tt) * ld_z + off_g + r]) : 0.f;
-        }
-        if (tid < nt) beta_s[tid] = dr_sigmoid(to_f(z[(size_t)(base + c0 + tid) * ld_z + off_b + h]));
-        for (int idx = tid; idx < nt * V; idx += NT) {
-            const int tt = idx / V, jj = idx - tt * V;
-            v_s[tt * V + jj] = to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + jj]);
-        }
-        __syncthreads();
-        // a thread takes one key channel of four rows at a time: a row of the factor is read once for the four
-        for (int idx = tid; idx < ((nt + 3) >> 2) * Dfull; idx += NT) {
-            const int tg = idx / Dfull, i = idx - tg * Dfull;
-            float a[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int idx = tid; idx < nt * Dfull; idx += NT) {
+            const int tt = idx / Dfull, i = idx - tt * Dfull;
+            const int at = tt * DP + (i / DPT) * PS + (i % DPT);
+            float kk = 0.f, qq = 0.f, gg = 1.f;
             if (i < D) {
-                const float* a1 = a1_s + (tg * 4) * rap;          // (rows beyond nt hold older numbers: never used)
-#pragma unroll 2
-                for (int r = 0; r < rap; r += 4) {
-                    float w4[4];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x)
-                        w4[x] = staged ? wa_s[(r + x) * D + i]
-                                       : (r + x < ra ? w_a2t[(size_t)(r + x) * H * D + h * D + i] : 0.f);
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const float4 c4 = *reinterpret_cast<const float4*>(a1 + k * rap + r);
-                        a[k] = fmaf(c4.x, w4[0], a[k]);
-                        a[k] = fmaf(c4.y, w4[1], a[k]);
-                        a[k] = fmaf(c4.z, w4[2], a[k]);
-                        a[k] = fmaf(c4.w, w4[3], a[k]);
-                    }
-                }
+                const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
+                qq = to_f(row[kvh * D + i]);
+                kk = to_f(row[G * D + kvh * D + i]);
+                const float a = to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i];
+                gg = expf(neg_a * dr_softplus(a));
             }
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int tt = tg * 4 + k;
-                if (tt >= nt) break;
-                const int at = tt * DP + (i / DPT) * PS + (i % DPT);
-                float kk = 0.f, qq = 0.f, gg = 1.f;
-                if (i < D) {
-                    const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
-                    qq = to_f(row[kvh * D + i]);
-                    kk = to_f(row[G * D + kvh * D + i]);
-                    gg = expf(neg_a * dr_softplus(a[k] + dt_bias[h * D + i]));
-                }
-                k_s[at] = kk;
-                q_s[at] = qq;
-                g_s[at] = gg;
-            }
+            k_s[at] = kk;
+            q_s[at] = qq;
+            g_s[at] = gg;
         }
         __syncthreads();
         for (int tt = wave; tt < nt; tt += n_waves) {          // unit vectors: a wave per row
@@ -185,7 +133,7 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
                 a3 = fmaf(st[ii + 3], k4.w, a3);
             }
             const float acc = dr_group_sum((a0 + a1) + (a2 + a3), RS);
-            const float u = beta_s[tt] * (v_s[tt * V + (live ? j : 0)] - acc);
+            const float u = beta_s[tt] * (v_s[tt * VB + (live ? jl : 0)] - acc);
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DPT; ii += 4) {
@@ -200,48 +148,9 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
                 o3 = fmaf(st[ii + 3], q4.w, o3);
             }
             const float o = dr_group_sum((o0 + o1) + (o2 + o3), RS);
-            if (live && rp == 0) o_s[tt * V + j] = o;
+            if (live && rp == 0) o_raw[(size_t)(base + c0 + tt) * H * V + h * V + j] = o;
         }
-        __syncthreads();
-        // ---- norm over the head's read-out (a wave per row), then weight and output gate: a thread takes one
-        // column of four rows at a time
-        for (int tt = wave; tt < nt; tt += n_waves) {
-            float ss = 0.f;
-            for (int jj = lane; jj < V; jj += 64) ss = fmaf(o_s[tt * V + jj], o_s[tt * V + jj], ss);
-            ss = wave_sum(ss);
-            if (lane == 0) rstd_s[tt] = 1.0f / sqrtf(ss / (float)V + eps);
-        }
-        __syncthreads();
-        for (int idx = tid; idx < ((nt + 3) >> 2) * V; idx += NT) {
-            const int tg = idx / V, jj = idx - tg * V;
-            float gt[4] = {0.f, 0.f, 0.f, 0.f};
-            const float* g1 = g1_s + (tg * 4) * rgp;
-#pragma unroll 2
-            for (int r = 0; r < rgp; r += 4) {
-                float w4[4];
-#pragma unroll
-                for (int x = 0; x < 4; ++x)
-                    w4[x] = staged ? wg_s[(r + x) * V + jj]
-                                   : (r + x < rg ? w_g2t[(size_t)(r + x) * H * V + h * V + jj] : 0.f);
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float4 c4 = *reinterpret_cast<const float4*>(g1 + k * rgp + r);
-                    gt[k] = fmaf(c4.x, w4[0], gt[k]);
-                    gt[k] = fmaf(c4.y, w4[1], gt[k]);
-                    gt[k] = fmaf(c4.z, w4[2], gt[k]);
-                    gt[k] = fmaf(c4.w, w4[3], gt[k]);
-                }
-            }
-            const float nw = norm_w[jj];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int tt = tg * 4 + k;
-                if (tt >= nt) break;
-                out[(size_t)(base + c0 + tt) * H * V + h * V + jj] =
-                    from_f<T>(o_s[tt * V + jj] * rstd_s[tt] * nw * dr_sigmoid(gt[k]));
-            }
-        }
-        __syncthreads();
+        __syncthreads();                                       // before the next chunk overwrites LDS
     }
 #pragma unroll
     for (int ii = 0; ii < DPT; ++ii) {
@@ -250,51 +159,65 @@ __global__ __launch_bounds__(512) void delta_rule_kernel(
     }
 }
 
-static size_t delta_rule_lds(int DPT, int RS, int V, int ra, int rg) {
-    const int rap = (ra + 3) & ~3, rgp = (rg + 3) & ~3;
-    return sizeof(float) * ((size_t)DR_TC * (3 * RS * (DPT + DR_PAD) + 2 * V + rap + rgp) + 2 * DR_TC);
+// out[t, h, :] = o[t, h, :] / sqrt(mean(o^2) + eps) * norm_w * sigmoid(c[t, h, :]): a wave per (row, head)
+template <typename T>
+__global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ gate,
+                                                        long long ld_gate, const float* __restrict__ norm_w, float eps,
+                                                        T* __restrict__ out, long long n_rows, int H, int V) {
+    const long long row = (long long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (row >= n_rows) return;
+    const int lane = threadIdx.x & 63;
+    const long long t = row / H;
+    const int h = (int)(row - t * H);
+    const float* o = o_raw + (size_t)row * V;
+    float ss = 0.f;
+    for (int jj = lane; jj < V; jj += 64) ss = fmaf(o[jj], o[jj], ss);
+    const float rstd = 1.0f / sqrtf(wave_sum(ss) / (float)V + eps);
+    for (int jj = lane; jj < V; jj += 64)
+        out[(size_t)row * V + jj] =
+            from_f<T>(o[jj] * rstd * norm_w[jj] * dr_sigmoid(to_f(gate[(size_t)t * ld_gate + (size_t)h * V + jj])));
 }
-// the low-rank factors' rows of one head beside that, if they fit
-static size_t delta_rule_staged(int D, int V, int ra, int rg) {
-    return sizeof(float) * ((size_t)((ra + 3) & ~3) * D + (size_t)((rg + 3) & ~3) * V);
-}
-#define DR_LDS_LIMIT (156 * 1024)
 
-// The split of a column's rows over lanes: RS lanes (a power of two) of DPT rows each.
-static bool delta_rule_plan(int D, int V, int* RS_out, int* DPT_out) {
-    if (D < 1 || V < 1 || V > 512 || D > 512) return false;
+// How a head's state is spread: RS lanes (a power of two) of DPT rows each to a column, VB columns a workgroup.
+static bool delta_rule_plan(int D, int V, int* RS_out, int* DPT_out, int* VB_out) {
+    if (D < 1 || V < 1 || D > 512 || V > 4096) return false;
     int RS = 8;
-    while (RS > 1 && (V * RS > 512 || (D + RS - 1) / RS < 8)) RS >>= 1;
+    while (RS > 1 && (D + RS - 1) / RS < 8) RS >>= 1;
     const int need = (D + RS - 1) / RS;
     int DPT = 4;
     while (DPT < need) DPT <<= 1;
     if (DPT > 64) return false;
+    int VB = 128 / RS;                              // two waves a workgroup
+    if (VB > V) VB = V;
     *RS_out = RS;
     *DPT_out = DPT;
+    *VB_out = VB;
     return true;
 }
 
-extern "C" int ra_delta_rule_fits(int D, int V, int ra, int rg) {
-    int RS, DPT;
-    if (!delta_rule_plan(D, V, &RS, &DPT) || ra < 0 || rg < 0) return 0;
-    return delta_rule_lds(DPT, RS, V, ra, rg) <= 160 * 1024 ? 1 : 0;
+static size_t delta_rule_lds(int DPT, int RS, int VB) {
+    return sizeof(float) * ((size_t)DR_TC * (3 * RS * (DPT + DR_PAD) + VB) + DR_TC);
+}
+
+extern "C" int ra_delta_rule_fits(int D, int V) {
+    int RS, DPT, VB;
+    if (!delta_rule_plan(D, V, &RS, &DPT, &VB)) return 0;
+    return delta_rule_lds(DPT, RS, VB) <= 160 * 1024 ? 1 : 0;
 }
 
 template <typename T>
 static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, size_t lds, const void* qkv, long long ld_qkv,
-                             const void* z, long long ld_z, int off_b, int off_a, int ra, int off_g, int rg,
-                             const float* w_a2t, const float* w_g2t, const float* A_log, const float* dt_bias,
-                             const float* norm_w, float eps, float* S, const int* cu_q, const int* slot_ids, void* out,
-                             int H, int G, int D, int V, int RS, int staged) {
+                             const void* b, long long ld_b, const void* ag, long long ld_ag, const float* A_log,
+                             const float* dt_bias, float* S, const int* cu_q, const int* slot_ids, float* o_raw, int H, int G,
+                             int D, int V, int RS, int VB) {
 #define DR_GO(DPT_)                                                                                               \
     do {                                                                                                          \
         if (lds > 64 * 1024 &&                                                                                    \
             hipFuncSetAttribute((const void*)delta_rule_kernel<T, DPT_>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                                 (int)lds) != hipSuccess)                                                          \
             return RA_ERR_LAUNCH;                                                                                 \
-        hipLaunchKernelGGL((delta_rule_kernel<T, DPT_>), grid, block, lds, st, (const T*)qkv, ld_qkv, (const T*)z, \
-                           ld_z, off_b, off_a, ra, off_g, rg, w_a2t, w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q,  \
-                           slot_ids, (T*)out, H, G, D, V, RS, staged);                                            \
+        hipLaunchKernelGGL((delta_rule_kernel<T, DPT_>), grid, block, lds, st, (const T*)qkv, ld_qkv, (const T*)b, ld_b, \
+                           (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, D, V, RS, VB);       \
     } while (0)
     switch (DPT) {
         case 4: DR_GO(4); break;
@@ -308,27 +231,40 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
     return ra_launch_status();
 }
 
-extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* z, long long ld_z, int off_b, int off_a, int ra,
-                             int off_g, int rg, const float* w_a2t, const float* w_g2t, const float* A_log,
-                             const float* dt_bias, const float* norm_w, float eps, float* S, const int* cu_q,
-                             const int* slot_ids, void* out, int n_seqs, int H, int G, int D, int V, int dtype,
-                             void* stream) {
-    if (n_seqs <= 0) return RA_OK;
-    int RS, DPT;
-    if (!delta_rule_plan(D, V, &RS, &DPT) || H < 1 || G < 1 || H % G || ra < 0 || rg < 0 || n_seqs > 65535) return RA_ERR_ARG;
-    if (ld_qkv < (long long)2 * G * D + (long long)H * V || off_b < 0 || off_a < 0 || off_g < 0) return RA_ERR_ARG;
-    if (ld_z < off_b + H || ld_z < off_a + ra || ld_z < off_g + rg) return RA_ERR_ARG;
-    size_t lds = delta_rule_lds(DPT, RS, V, ra, rg);
+// qkv [T, 2 G D + H V] rows; b: rows whose first H columns are the heads' beta (before the sigmoid); ag [T, H D + H V];
+// S fp32 [slots, H, D, V]; o_raw fp32 [T, H V] scratch; out [T, H V].
+extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, long long ld_b, const void* ag,
+                             long long ld_ag, const float* A_log, const float* dt_bias, const float* norm_w, float eps,
+                             float* S, const int* cu_q, const int* slot_ids, float* o_raw, void* out, int n_seqs,
+                             int T_tokens, int H, int G, int D, int V, int dtype, void* stream) {
+    if (n_seqs <= 0 || T_tokens <= 0) return RA_OK;
+    int RS, DPT, VB;
+    if (!delta_rule_plan(D, V, &RS, &DPT, &VB) || H < 1 || G < 1 || H % G || n_seqs > 65535) return RA_ERR_ARG;
+    if (ld_qkv < (long long)2 * G * D + (long long)H * V || ld_b < H || ld_ag < (long long)H * D + (long long)H * V)
+        return RA_ERR_ARG;
+    if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
+    const size_t lds = delta_rule_lds(DPT, RS, VB);
     if (lds > 160 * 1024) return RA_ERR_ARG;
-    const int staged = lds + delta_rule_staged(D, V, ra, rg) <= DR_LDS_LIMIT ? 1 : 0;
-    if (staged) lds += delta_rule_staged(D, V, ra, rg);
-    dim3 grid(H, n_seqs), block(((V * RS + 63) / 64) * 64);
+    const int col_blocks = (V + VB - 1) / VB;
+    if ((long long)H * col_blocks > 0x7fffffffLL) return RA_ERR_ARG;
+    dim3 grid(H * col_blocks, n_seqs), block(((VB * RS + 63) / 64) * 64);
     hipStream_t st = (hipStream_t)stream;
+    int rc;
     if (dtype == RA_DTYPE_F32)
-        return delta_rule_launch<float>(st, DPT, grid, block, lds, qkv, ld_qkv, z, ld_z, off_b, off_a, ra, off_g, rg, w_a2t,
-                                        w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids, out, H, G, D, V, RS, staged);
-    if (dtype == RA_DTYPE_BF16)
-        return delta_rule_launch<bf16>(st, DPT, grid, block, lds, qkv, ld_qkv, z, ld_z, off_b, off_a, ra, off_g, rg, w_a2t,
-                                       w_g2t, A_log, dt_bias, norm_w, eps, S, cu_q, slot_ids, out, H, G, D, V, RS, staged);
-    return RA_ERR_ARG;
+        rc = delta_rule_launch<float>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
+                                      slot_ids, o_raw, H, G, D, V, RS, VB);
+    else
+        rc = delta_rule_launch<bf16>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
+                                     slot_ids, o_raw, H, G, D, V, RS, VB);
+    if (rc != RA_OK) return rc;
+    const long long n_rows = (long long)T_tokens * H;
+    dim3 ogrid((unsigned)((n_rows + 3) / 4)), oblock(256);
+    const long long gate_off = (long long)H * D;
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(delta_out_kernel<float>, ogrid, oblock, 0, st, o_raw, (const float*)ag + gate_off, ld_ag, norm_w,
+                           eps, (float*)out, n_rows, H, V);
+    else
+        hipLaunchKernelGGL(delta_out_kernel<bf16>, ogrid, oblock, 0, st, o_raw, (const bf16*)ag + gate_off, ld_ag, norm_w,
+                           eps, (bf16*)out, n_rows, H, V);
+    return ra_launch_status();
 }

@@ -72,8 +72,8 @@ def _declare(lib):
         "ra_gemm_sweep_norm_bf16": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, F, I, I, P],
         "ra_causal_conv": [P, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
-        "ra_delta_rule": [P, L, P, L, I, I, I, I, I, P, P, P, P, P, F, P, P, P, P, I, I, I, I, I, I, P],
-        "ra_delta_rule_fits": [I, I, I, I],
+        "ra_delta_rule": [P, L, P, L, P, L, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "ra_delta_rule_fits": [I, I],
         "ra_token_side": [P, P, P, P, L, I, P, P, P, F, I, I, I, I, P],
         "ra_relu_sq": [P, L, I, P],
         "ra_add_bias": [P, P, L, I, I, P],
@@ -419,40 +419,39 @@ class HipOps:
             "causal_conv")
         return out
 
-    def delta_rule_fits(self, D, V, rank_a, rank_g):
-        return bool(self.lib.ra_delta_rule_fits(int(D), int(V), int(rank_a), int(rank_g)))
+    def delta_rule_fits(self, D, V):
+        return bool(self.lib.ra_delta_rule_fits(int(D), int(V)))
 
-    def delta_rule(self, qkv, z, off_b, off_a, rank_a, off_g, rank_g, w_a2t, w_g2t, a_log, dt_bias, norm_w, eps,
-                   state, step, out, H, G, D, V):
-        """The gated delta rule with a decay per key channel over the step's rows, with everything around it
-        (unit q and k, beta, the decay's and the output gate's low-rank second factors, the norm of the
-        read-out) in the one kernel. qkv: [T, 2 G D + H V] after the short convolution; z: the fused input
-        projection's rows (beta at column off_b, the low-rank first factors at off_a and off_g);
-        state: fp32 [slots, H, D, V], updated in place; out: [T, H V]."""
+    def delta_rule(self, qkv, beta, ag, a_log, dt_bias, norm_w, eps, state, step, out, H, G, D, V):
+        """The gated delta rule with a decay per key channel over the step's rows, with what surrounds it in
+        32-bit (unit q and k, sigmoid of beta, softplus and exponentials of the decay, the norm of the read-out
+        and its gate). qkv: [T, 2 G D + H V] after the short convolution; beta: [T, H] before the sigmoid;
+        ag: [T, H D + H V], the decay's and the output gate's projections; each may be a column slice of wider
+        rows. state: fp32 [slots, H, D, V], updated in place; out: [T, H V]."""
         ld_qkv = self._want_rows(qkv, "delta-rule q/k/v")
-        ld_z = self._want_rows(z, "delta-rule projections", qkv.dtype)
+        ld_b = self._want_rows(beta, "delta-rule beta", qkv.dtype)
+        ld_ag = self._want_rows(ag, "delta-rule decay and gate projections", qkv.dtype)
         self._want(out, "delta-rule output", qkv.dtype, 2)
         self._want(state, "delta-rule state", torch.float32, 4)
         T = qkv.shape[0]
-        for t, name, shape in ((w_a2t, "decay factor", (rank_a, H * D)), (w_g2t, "gate factor", (rank_g, H * V)),
-                               (a_log, "A_log", (H,)), (dt_bias, "dt_bias", (H * D,)), (norm_w, "norm weight", (V,))):
+        for t, name, shape in ((a_log, "A_log", (H,)), (dt_bias, "dt_bias", (H * D,)), (norm_w, "norm weight", (V,))):
             self._want(t, name, torch.float32)
             if tuple(t.shape) != shape:
                 raise KernelError(f"delta_rule: {name} is {tuple(t.shape)}, wanted {shape}")
-        if qkv.shape[1] != 2 * G * D + H * V or tuple(out.shape) != (T, H * V) or z.shape[0] != T or T != step.n_tokens \
-                or tuple(state.shape[1:]) != (H, D, V) or H % G:
-            raise KernelError(f"delta_rule: qkv {tuple(qkv.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)}, "
-                              f"state {tuple(state.shape)}, {H} heads over {G} of {D} x {V}, step of {step.n_tokens}")
-        if max(off_b + H, off_a + rank_a, off_g + rank_g) > z.shape[1] or min(off_b, off_a, off_g) < 0:
-            raise KernelError(f"delta_rule: columns {off_b}, {off_a}, {off_g} beyond rows of {z.shape[1]}")
+        if qkv.shape[1] != 2 * G * D + H * V or tuple(out.shape) != (T, H * V) or tuple(beta.shape) != (T, H) \
+                or tuple(ag.shape) != (T, H * D + H * V) or T != step.n_tokens or tuple(state.shape[1:]) != (H, D, V) or H % G:
+            raise KernelError(f"delta_rule: qkv {tuple(qkv.shape)}, beta {tuple(beta.shape)}, ag {tuple(ag.shape)}, "
+                              f"out {tuple(out.shape)}, state {tuple(state.shape)}, {H} heads over {G} of {D} x {V}, "
+                              f"step of {step.n_tokens}")
         if max(step.slot_ids_host, default=0) >= state.shape[0]:
             raise KernelError("delta_rule: a request's slot lies beyond the state's rows")
-        if not self.delta_rule_fits(D, V, rank_a, rank_g):
-            raise KernelError(f"delta_rule: heads of {D} x {V} with ranks {rank_a}, {rank_g} are beyond the kernel")
+        if not self.delta_rule_fits(D, V):
+            raise KernelError(f"delta_rule: heads of {D} x {V} are beyond the kernel")
+        o_raw = torch.empty(T, H * V, dtype=torch.float32, device=self.device)
         self._check(self.lib.ra_delta_rule(
-            _ptr(qkv), ld_qkv, _ptr(z), ld_z, off_b, off_a, rank_a, off_g, rank_g, _ptr(w_a2t), _ptr(w_g2t), _ptr(a_log),
-            _ptr(dt_bias), _ptr(norm_w), float(eps), _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(out),
-            step.n_seqs, H, G, D, V, _code(qkv.dtype), self._stream()), "delta_rule")
+            _ptr(qkv), ld_qkv, _ptr(beta), ld_b, _ptr(ag), ld_ag, _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), float(eps),
+            _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out), step.n_seqs, T, H, G, D, V,
+            _code(qkv.dtype), self._stream()), "delta_rule")
         return out
 
     def token_side(self, h, delta, token_ids, table, offset, gate, proj, weight, eps):

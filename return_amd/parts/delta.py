@@ -11,9 +11,10 @@ For head h with its q/k head h // (heads / kv_heads), token by token:
 Everything from the unit vectors to the norm of o is 32-bit. Kept between steps per request: the
 last taps-1 inputs of the three convolutions and S.
 
-One product forms q, k, v, b and the first factors of the two low-rank maps (the weights stacked,
-rows padded to a multiple of 16); the convolution reads its columns of that result in place; the
-recurrence kernel reads the rest and applies the second factors itself.
+Three products in front: q, k, v and b as one (the weights stacked, rows padded to a multiple of
+16), the first factors of the two low-rank maps as one, and their second factors as one (a matrix of
+two blocks on its diagonal); the convolution reads its columns of the first result in place, the
+recurrence kernels read the rest.
 """
 from __future__ import annotations
 
@@ -67,22 +68,27 @@ class ChannelDeltaMixer:
         self.ra, self.rg = tensors["a1_proj"].shape[0], tensors["g1_proj"].shape[0]
         if tensors["a2_proj"].shape[1] != self.ra or tensors["g2_proj"].shape[1] != self.rg:
             raise ValueError("the two factors of a low-rank map differ in their inner size")
-        if hasattr(rt.ops, "delta_rule_fits") and not rt.ops.delta_rule_fits(self.D, self.V, self.ra, self.rg):
-            raise ValueError(f"heads of {self.D} x {self.V} with low-rank maps of {self.ra} and {self.rg} are beyond "
-                             "the delta-rule kernel")
         self.c_conv = 2 * self.G * self.D + self.H * self.V
-        self.off_b = self.c_conv
-        self.off_a = self.off_b + self.H
-        self.off_g = self.off_a + self.ra
-        used = self.off_g + self.rg
-        rows = [rt.matrix(tensors[n]) for n in ("q_proj", "k_proj", "v_proj", "b_proj", "a1_proj", "g1_proj")]
-        pad = -used % 16
-        if pad:
-            rows.append(torch.zeros(pad, W, dtype=rt.dtype, device=rt.device))
-        self.w_in = rt.product(torch.cat(rows, dim=0).contiguous())
+        if hasattr(rt.ops, "delta_rule_fits") and not rt.ops.delta_rule_fits(self.D, self.V):
+            raise ValueError(f"heads of {self.D} x {self.V} are beyond the delta-rule kernel")
+
+        def stacked(rows, width):
+            """Matrices one under the other, rows filled up with zeros to a multiple of 16."""
+            pad = -sum(r.shape[0] for r in rows) % 16
+            if pad:
+                rows = rows + [torch.zeros(pad, width, dtype=rt.dtype, device=rt.device)]
+            return torch.cat(rows, dim=0).contiguous()
+
+        self.w_in = rt.product(stacked([rt.matrix(tensors[n]) for n in ("q_proj", "k_proj", "v_proj", "b_proj")], W))
+        self.w_low = rt.product(stacked([rt.matrix(tensors["a1_proj"]), rt.matrix(tensors["g1_proj"])], W))
+        # [a | c] = [a1 | g1 | 0] @ [[A2, 0], [0, G2], [0, 0]]^T: the two second factors as one product
+        r_in = self.w_low.shape[0]
+        n_a, n_c = self.H * self.D, self.H * self.V
+        second = torch.zeros(n_a + n_c, r_in, dtype=rt.dtype, device=rt.device)
+        second[:n_a, :self.ra] = rt.matrix(tensors["a2_proj"])
+        second[n_a:, self.ra:self.ra + self.rg] = rt.matrix(tensors["g2_proj"])
+        self.w_second = rt.product(second)
         self.w_conv = torch.cat([rt.vector32(tensors[n]) for n in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
-        self.w_a2t = rt.vector32(tensors["a2_proj"]).t().contiguous()          # [ra, H*D]
-        self.w_g2t = rt.vector32(tensors["g2_proj"]).t().contiguous()          # [rg, H*V]
         self.a_log = rt.vector32(tensors["A_log"])
         self.dt_bias = rt.vector32(tensors["dt_bias"])
         self.w_norm = rt.vector32(tensors["o_norm"])
@@ -97,13 +103,13 @@ class ChannelDeltaMixer:
         if not write_cache:
             raise ValueError("a delta-rule mixer advances its state with every call; it cannot only read it")
         T = x.shape[0]
-        z = ops.linear(x, self.w_in)                                           # [T, q | k | v | b | a1 | g1 | pad]
+        z = ops.linear(x, self.w_in)                                           # [T, q | k | v | b | pad]
+        ag = ops.linear(ops.linear(x, self.w_low), self.w_second)              # [T, decay H*D | gate H*V]
         qkv = rt.empty(T, self.c_conv)
         ops.causal_conv(z[:, :self.c_conv], self.w_conv, cache.tensors["conv"], step, qkv, silu=True)
         o = rt.empty(T, self.H * self.V)
-        ops.delta_rule(qkv, z, self.off_b, self.off_a, self.ra, self.off_g, self.rg, self.w_a2t, self.w_g2t,
-                       self.a_log, self.dt_bias, self.w_norm, self.eps, cache.tensors["S"], step, o,
-                       self.H, self.G, self.D, self.V)
+        ops.delta_rule(qkv, z[:, self.c_conv:self.c_conv + self.H], ag, self.a_log, self.dt_bias, self.w_norm, self.eps,
+                       cache.tensors["S"], step, o, self.H, self.G, self.D, self.V)
         return ops.linear(o, self.w_o)
 
 

@@ -129,7 +129,8 @@ def test_delta_rule_in_pieces_equals_the_plain_recurrence():
     # what the kernel is given: the rows after convolution and activation, and the other projections
     silu = lambda z: z * torch.sigmoid(z)
     qkv = torch.cat([silu(h @ w["q"].T), silu(h @ w["k"].T), silu(h @ w["v"].T)], dim=1).float()
-    z = torch.cat([h @ w["b"].T, h @ w["a1"].T, h @ w["g1"].T], dim=1).float()
+    beta = (h @ w["b"].T).float()
+    ag = torch.cat([(h @ w["a1"].T) @ w["a2"].T, (h @ w["g1"].T) @ w["g2"].T], dim=1).float()
     ops = TorchOps("cpu")
     state = torch.randn(3, H, D, V, generator=g)
     state[2].zero_()
@@ -137,9 +138,8 @@ def test_delta_rule_in_pieces_equals_the_plain_recurrence():
     at = 0
     for n in (4, 1, 1, 2, 11):
         step = _Step([n], [2])
-        ops.delta_rule(qkv[at:at + n], z[at:at + n], 0, H, r, H + r, r, w["a2"].T.float().contiguous(),
-                       w["g2"].T.float().contiguous(), w["A_log"].float(), w["dt_bias"].float(), w["norm"].float(), 1e-5,
-                       state, step, out[at:at + n], H, G, D, V)
+        ops.delta_rule(qkv[at:at + n], beta[at:at + n], ag[at:at + n], w["A_log"].float(), w["dt_bias"].float(),
+                       w["norm"].float(), 1e-5, state, step, out[at:at + n], H, G, D, V)
         at += n
     torch.testing.assert_close(out.double(), want, atol=2e-5, rtol=1e-4)
 

@@ -79,17 +79,17 @@ def test_causal_conv(ops, ref, dtype, C, taps, q_lens, flags):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,D,V,ra,rg,q_lens", [
-    (4, 2, 16, 32, 8, 8, [1, 1, 1]), (3, 3, 12, 20, 6, 3, [5, 1, 33]), (2, 1, 64, 64, 24, 24, [40]),
-    (6, 2, 20, 12, 3, 5, [2, 17]), (1, 1, 64, 48, 2, 2, [1, 19]), (2, 2, 128, 128, 16, 8, [1, 21]),
-    (2, 1, 8, 256, 4, 4, [3]), (2, 2, 256, 16, 4, 4, [1, 4])])
-def test_delta_rule(ops, ref, dtype, H, G, D, V, ra, rg, q_lens):
+@pytest.mark.parametrize("H,G,D,V,q_lens", [
+    (4, 2, 16, 32, [1, 1, 1]), (3, 3, 12, 20, [5, 1, 33]), (2, 1, 64, 64, [40]), (6, 2, 20, 12, [2, 17]),
+    (1, 1, 64, 48, [1, 19]), (2, 2, 128, 128, [1, 70]), (2, 1, 8, 256, [3]), (2, 2, 256, 16, [1, 4]), (5, 5, 7, 3, [9])])
+def test_delta_rule(ops, ref, dtype, H, G, D, V, q_lens):
+    """Two steps in a row over slots that hold something; the inputs are column slices of wider rows."""
     n = len(q_lens)
     T = sum(q_lens)
     slots = torch.randperm(n + 1, generator=torch.Generator().manual_seed(n)).tolist()[:n]
     qkv = rnd(T, 2 * G * D + H * V, dtype=dtype, seed=1)
-    z = rnd(T, 16 + H + ra + rg + 5, dtype=dtype, seed=2)
-    w_a2t, w_g2t = rnd(ra, H * D, seed=3, scale=0.5), rnd(rg, H * V, seed=4, scale=0.5)
+    z = rnd(T, 24 + H, dtype=dtype, seed=2)
+    ag = rnd(T, H * D + H * V + 8, dtype=dtype, seed=3)[:, :H * D + H * V]
     a_log, dt_bias, norm_w = rnd(H, seed=5), rnd(H * D, seed=6) - 1.0, 1 + rnd(V, seed=7, scale=0.1)
     state_a = rnd(n + 1, H, D, V, seed=8, scale=0.3)
     state_b = state_a.clone()
@@ -97,7 +97,7 @@ def test_delta_rule(ops, ref, dtype, H, G, D, V, ra, rg, q_lens):
         step = state_step(q_lens, slots)
         a = torch.empty(T, H * V, dtype=dtype, device=DEV)
         b = torch.empty_like(a)
-        args = (qkv, z, 16, 16 + H, ra, 16 + H + ra, rg, w_a2t, w_g2t, a_log, dt_bias, norm_w, 1e-5)
+        args = (qkv, z[:, 16:16 + H], ag, a_log, dt_bias, norm_w, 1e-5)
         ops.delta_rule(*args, state_a, step, a, H, G, D, V)
         ref.delta_rule(*args, state_b, step, b, H, G, D, V)
         torch.testing.assert_close(a.float(), b.float(), **tol(dtype))

@@ -205,11 +205,10 @@ class TorchOps:
                 tail[slots[s]] = seq[-(taps - 1):].to(tail.dtype)
         return out
 
-    def delta_rule_fits(self, D, V, rank_a, rank_g):
+    def delta_rule_fits(self, D, V):
         return True
 
-    def delta_rule(self, qkv, z, off_b, off_a, rank_a, off_g, rank_g, w_a2t, w_g2t, a_log, dt_bias, norm_w, eps,
-                   state, step, out, H, G, D, V):
+    def delta_rule(self, qkv, beta, ag, a_log, dt_bias, norm_w, eps, state, step, out, H, G, D, V):
         cu, slots = step.cu_q_host, step.slot_ids_host
         T = qkv.shape[0]
         q = qkv[:, :G * D].float().view(T, G, D)
@@ -217,10 +216,10 @@ class TorchOps:
         v = qkv[:, 2 * G * D:].float().view(T, H, V)
         q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6) * D ** -0.5
         k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
-        beta = torch.sigmoid(z[:, off_b:off_b + H].float())
-        a = z[:, off_a:off_a + rank_a].float() @ w_a2t + dt_bias
+        beta = torch.sigmoid(beta.float())
+        a = ag[:, :H * D].float() + dt_bias
         g = torch.exp(-torch.exp(a_log)[None, :, None] * torch.nn.functional.softplus(a).view(T, H, D))
-        gate = torch.sigmoid(z[:, off_g:off_g + rank_g].float() @ w_g2t).view(T, H, V)
+        gate = torch.sigmoid(ag[:, H * D:].float()).view(T, H, V)
         rep = H // G
         for s in range(step.n_seqs):
             S = state[slots[s]]                               # [H, D, V], updated in place
