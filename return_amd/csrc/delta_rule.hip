@@ -26,6 +26,13 @@
 
 __device__ __forceinline__ float dr_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
 __device__ __forceinline__ float dr_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+// The decay exp(-A softplus(x)) by the hardware's exponential and logarithm (relative error about 1e-6; where
+// e^x is tiny, log(1 + e^x) is off by at most one rounding of 1, 6e-8, and so is the decay): this runs once per
+// token and key channel inside the walk over the tokens, where the exact routines' hundred instructions count.
+__device__ __forceinline__ float dr_decay(float neg_a, float x) {
+    const float sp = x > 20.f ? x : __logf(1.f + __expf(x));
+    return __expf(neg_a * sp);
+}
 
 // Sum over the RS (1, 2, 4 or 8) neighbouring lanes that share a column, in every one of them, by
 // data-parallel moves inside a row of 16 lanes: partner lane ^ 1, then lane ^ 2, then the other quad
@@ -40,8 +47,10 @@ __device__ __forceinline__ float dr_group_sum(float v, int RS) {
     return v;
 }
 
+// (one or two waves a SIMD: the walk is a chain of dependent steps, and registers for the next token's operands
+// serve it better than more waves would)
 template <typename T, int DPT>
-__global__ __launch_bounds__(256) void delta_rule_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) void delta_rule_kernel(
     const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ b, long long ld_b, const T* __restrict__ ag,
     long long ld_ag, const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ S,
     const int* __restrict__ cu_q, const int* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int D, int V,
@@ -82,20 +91,32 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
             const int tt = idx / VB, jj = idx - tt * VB;
             v_s[idx] = j0 + jj < V ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
         }
-        for (int idx = tid; idx < nt * Dfull; idx += NT) {
-            const int tt = idx / Dfull, i = idx - tt * Dfull;
-            const int at = tt * DP + (i / DPT) * PS + (i % DPT);
-            float kk = 0.f, qq = 0.f, gg = 1.f;
-            if (i < D) {
-                const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
-                qq = to_f(row[kvh * D + i]);
-                kk = to_f(row[G * D + kvh * D + i]);
-                const float a = to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i];
-                gg = expf(neg_a * dr_softplus(a));
+        // (four elements a thread at a time: their loads are on their way together)
+        for (int idx0 = tid; idx0 < nt * Dfull; idx0 += 4 * NT) {
+            float kk[4], qq[4], aa[4];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int idx = idx0 + x * NT;
+                const int tt = idx / Dfull, i = idx - tt * Dfull;
+                kk[x] = qq[x] = 0.f;
+                aa[x] = 0.f;
+                if (idx < nt * Dfull && i < D) {
+                    const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
+                    qq[x] = to_f(row[kvh * D + i]);
+                    kk[x] = to_f(row[G * D + kvh * D + i]);
+                    aa[x] = to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i];
+                }
             }
-            k_s[at] = kk;
-            q_s[at] = qq;
-            g_s[at] = gg;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                const int idx = idx0 + x * NT;
+                if (idx >= nt * Dfull) break;
+                const int tt = idx / Dfull, i = idx - tt * Dfull;
+                const int at = tt * DP + (i / DPT) * PS + (i % DPT);
+                k_s[at] = kk[x];
+                q_s[at] = qq[x];
+                g_s[at] = i < D ? dr_decay(neg_a, aa[x]) : 1.f;
+            }
         }
         __syncthreads();
         for (int tt = wave; tt < nt; tt += n_waves) {          // unit vectors: a wave per row
@@ -115,40 +136,58 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
         }
         __syncthreads();
         // ---- the recurrence over the chunk
+        // (a token's k, g and q are read from LDS while the token before it is worked on)
+        float kreg[DPT], greg[DPT], qreg[DPT];
+#pragma unroll
+        for (int ii = 0; ii < DPT; ii += 4) {
+            *reinterpret_cast<float4*>(kreg + ii) = *reinterpret_cast<const float4*>(k_s + rp * PS + ii);
+            *reinterpret_cast<float4*>(greg + ii) = *reinterpret_cast<const float4*>(g_s + rp * PS + ii);
+            *reinterpret_cast<float4*>(qreg + ii) = *reinterpret_cast<const float4*>(q_s + rp * PS + ii);
+        }
         for (int tt = 0; tt < nt; ++tt) {
-            const float* kr = k_s + tt * DP + rp * PS;
-            const float* qr = q_s + tt * DP + rp * PS;
-            const float* gr = g_s + tt * DP + rp * PS;
-            float kreg[DPT];
+            const int nx = min(tt + 1, nt - 1);
+            const float* kr = k_s + nx * DP + rp * PS;
+            const float* qr = q_s + nx * DP + rp * PS;
+            const float* gr = g_s + nx * DP + rp * PS;
+            float kn[DPT], gn[DPT], qn[DPT];
+#pragma unroll
+            for (int ii = 0; ii < DPT; ii += 4) {
+                *reinterpret_cast<float4*>(kn + ii) = *reinterpret_cast<const float4*>(kr + ii);
+                *reinterpret_cast<float4*>(gn + ii) = *reinterpret_cast<const float4*>(gr + ii);
+                *reinterpret_cast<float4*>(qn + ii) = *reinterpret_cast<const float4*>(qr + ii);
+            }
+            const float beta = beta_s[tt], vv = v_s[tt * VB + (live ? jl : 0)];
             float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;         // four chains, so that no sum waits for the one before
 #pragma unroll
             for (int ii = 0; ii < DPT; ii += 4) {
-                const float4 k4 = *reinterpret_cast<const float4*>(kr + ii);
-                const float4 g4 = *reinterpret_cast<const float4*>(gr + ii);
-                kreg[ii] = k4.x; kreg[ii + 1] = k4.y; kreg[ii + 2] = k4.z; kreg[ii + 3] = k4.w;
-                st[ii] *= g4.x; st[ii + 1] *= g4.y; st[ii + 2] *= g4.z; st[ii + 3] *= g4.w;
-                a0 = fmaf(st[ii], k4.x, a0);
-                a1 = fmaf(st[ii + 1], k4.y, a1);
-                a2 = fmaf(st[ii + 2], k4.z, a2);
-                a3 = fmaf(st[ii + 3], k4.w, a3);
+                st[ii] *= greg[ii]; st[ii + 1] *= greg[ii + 1]; st[ii + 2] *= greg[ii + 2]; st[ii + 3] *= greg[ii + 3];
+                a0 = fmaf(st[ii], kreg[ii], a0);
+                a1 = fmaf(st[ii + 1], kreg[ii + 1], a1);
+                a2 = fmaf(st[ii + 2], kreg[ii + 2], a2);
+                a3 = fmaf(st[ii + 3], kreg[ii + 3], a3);
             }
             const float acc = dr_group_sum((a0 + a1) + (a2 + a3), RS);
-            const float u = beta_s[tt] * (v_s[tt * VB + (live ? jl : 0)] - acc);
+            const float u = beta * (vv - acc);
             float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DPT; ii += 4) {
-                const float4 q4 = *reinterpret_cast<const float4*>(qr + ii);
                 st[ii] = fmaf(kreg[ii], u, st[ii]);
                 st[ii + 1] = fmaf(kreg[ii + 1], u, st[ii + 1]);
                 st[ii + 2] = fmaf(kreg[ii + 2], u, st[ii + 2]);
                 st[ii + 3] = fmaf(kreg[ii + 3], u, st[ii + 3]);
-                o0 = fmaf(st[ii], q4.x, o0);
-                o1 = fmaf(st[ii + 1], q4.y, o1);
-                o2 = fmaf(st[ii + 2], q4.z, o2);
-                o3 = fmaf(st[ii + 3], q4.w, o3);
+                o0 = fmaf(st[ii], qreg[ii], o0);
+                o1 = fmaf(st[ii + 1], qreg[ii + 1], o1);
+                o2 = fmaf(st[ii + 2], qreg[ii + 2], o2);
+                o3 = fmaf(st[ii + 3], qreg[ii + 3], o3);
             }
             const float o = dr_group_sum((o0 + o1) + (o2 + o3), RS);
             if (live && rp == 0) o_raw[(size_t)(base + c0 + tt) * H * V + h * V + j] = o;
+#pragma unroll
+            for (int ii = 0; ii < DPT; ++ii) {
+                kreg[ii] = kn[ii];
+                greg[ii] = gn[ii];
+                qreg[ii] = qn[ii];
+            }
         }
         __syncthreads();                                       // before the next chunk overwrites LDS
     }
