@@ -81,18 +81,18 @@ __global__ __launch_bounds__(TS_THREADS) void token_side_kernel(
 // forms its product with all R stream rows, each lane eight columns at a time, so that all of a row's
 // loads are on their way at once and a gate row is read once for R rows; then a thread forms its columns of
 // y for all R rows from one read of the projection's row.
-template <int R>
-__global__ __launch_bounds__(TS_THREADS) void token_side_bf16x8_kernel(
+template <int R, int NTH>
+__global__ __launch_bounds__(NTH) void token_side_bf16x8_kernel(
     float* __restrict__ h, const bf16* __restrict__ delta, const int* __restrict__ ids, const bf16* __restrict__ table,
     long long ld_table, int off, const bf16* __restrict__ gate, const bf16* __restrict__ proj,
     const float* __restrict__ w, float eps, int T_tokens, int H, int S) {
     extern __shared__ __attribute__((aligned(16))) float ts_smem[];
     float* x_s = ts_smem;                        // [R][H]
     float* g_s = x_s + (size_t)R * H;            // [R][S]
-    float* red = g_s + R * S;                    // [R][4]
+    float* red = g_s + R * S;                    // [R][waves]
     const int t0 = blockIdx.x * R, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int rows = min(R, T_tokens - t0);
-    for (int idx = tid * 4; idx < R * H; idx += TS_THREADS * 4) {
+    for (int idx = tid * 4; idx < R * H; idx += NTH * 4) {
         const int rr = idx / H, c = idx - rr * H;
         float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
         if (rr < rows) {
@@ -106,7 +106,7 @@ __global__ __launch_bounds__(TS_THREADS) void token_side_bf16x8_kernel(
         *reinterpret_cast<float4*>(x_s + idx) = v;
     }
     __syncthreads();
-    for (int r = wave; r < S; r += TS_THREADS / 64) {
+    for (int r = wave; r < S; r += (NTH / 64)) {
         float a[R];
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) a[rr] = 0.f;
@@ -137,13 +137,13 @@ __global__ __launch_bounds__(TS_THREADS) void token_side_bf16x8_kernel(
         }
     }
     __syncthreads();
-    float y[R][TS_MAX_CPT / 2];                  // H <= 256 * 16 in this form
+    float y[R][(4096 / NTH)];                  // H <= 4096 in this form
     float ss[R];
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) ss[rr] = 0.f;
 #pragma unroll
-    for (int i = 0; i < TS_MAX_CPT / 2; ++i) {
-        const int c = tid + i * TS_THREADS;
+    for (int i = 0; i < (4096 / NTH); ++i) {
+        const int c = tid + i * NTH;
 #pragma unroll
         for (int rr = 0; rr < R; ++rr) y[rr][i] = 0.f;
         if (c < H) {
@@ -165,32 +165,33 @@ __global__ __launch_bounds__(TS_THREADS) void token_side_bf16x8_kernel(
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
         const float v = wave_sum(ss[rr]);
-        if (lane == 0) red[rr * 4 + wave] = v;
+        if (lane == 0) red[rr * (NTH / 64) + wave] = v;
     }
     __syncthreads();
 #pragma unroll
     for (int rr = 0; rr < R; ++rr) {
         if (rr >= rows) break;
-        const float tot = (red[rr * 4] + red[rr * 4 + 1]) + (red[rr * 4 + 2] + red[rr * 4 + 3]);
+        float tot = 0.f;
+        for (int wv = 0; wv < NTH / 64; ++wv) tot += red[rr * (NTH / 64) + wv];      // (the same order in every thread)
         const float rstd = 1.0f / sqrtf(tot / (float)H + eps);
 #pragma unroll
-        for (int i = 0; i < TS_MAX_CPT / 2; ++i) {
-            const int c = tid + i * TS_THREADS;
+        for (int i = 0; i < (4096 / NTH); ++i) {
+            const int c = tid + i * NTH;
             if (c < H) h[(size_t)(t0 + rr) * H + c] = x_s[(size_t)rr * H + c] + y[rr][i] * rstd * w[c];
         }
     }
 }
 
-template <int R>
+template <int R, int NTH>
 static int token_side_x8_launch(hipStream_t st, float* h, const void* delta, const int* ids, const void* table,
                                 long long ld_table, int off, const void* gate, const void* proj, const float* w, float eps,
                                 int T_tokens, int H, int S) {
-    const size_t lds = sizeof(float) * ((size_t)R * H + (size_t)R * S + R * 4);
+    const size_t lds = sizeof(float) * ((size_t)R * H + (size_t)R * S + R * (NTH / 64));
     if (lds > 64 * 1024 &&
-        hipFuncSetAttribute((const void*)token_side_bf16x8_kernel<R>, hipFuncAttributeMaxDynamicSharedMemorySize,
+        hipFuncSetAttribute((const void*)token_side_bf16x8_kernel<R, NTH>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)lds) != hipSuccess)
         return RA_ERR_LAUNCH;
-    hipLaunchKernelGGL((token_side_bf16x8_kernel<R>), dim3((T_tokens + R - 1) / R), dim3(TS_THREADS), lds, st, h,
+    hipLaunchKernelGGL((token_side_bf16x8_kernel<R, NTH>), dim3((T_tokens + R - 1) / R), dim3(NTH), lds, st, h,
                        (const bf16*)delta, ids, (const bf16*)table, ld_table, off, (const bf16*)gate, (const bf16*)proj, w,
                        eps, T_tokens, H, S);
     return ra_launch_status();
@@ -203,11 +204,14 @@ extern "C" int ra_token_side(float* h, const void* delta, const int* ids, const 
     if (S < 1 || S > TS_MAX_S || H < 1 || H > TS_THREADS * TS_MAX_CPT || off < 0 || ld_table < off + S) return RA_ERR_ARG;
     dim3 grid(T_tokens), block(TS_THREADS);
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == RA_DTYPE_BF16 && H % 8 == 0 && S % 8 == 0 && H <= TS_THREADS * TS_MAX_CPT / 2 && ld_table >= 0) {
+    if (dtype == RA_DTYPE_BF16 && H % 8 == 0 && S % 8 == 0 && H <= 4096) {
         // many rows: four a workgroup, so that the two matrices are read once for four rows
         if (T_tokens >= 256)
-            return token_side_x8_launch<4>(st, h, delta, ids, table, ld_table, off, gate, proj, w, eps, T_tokens, H, S);
-        return token_side_x8_launch<1>(st, h, delta, ids, table, ld_table, off, gate, proj, w, eps, T_tokens, H, S);
+            return token_side_x8_launch<4, 256>(st, h, delta, ids, table, ld_table, off, gate, proj, w, eps, T_tokens, H, S);
+        // few rows: sixteen waves a row, so that a row's loads are spread over four times the threads
+        if (T_tokens <= 64)
+            return token_side_x8_launch<1, 1024>(st, h, delta, ids, table, ld_table, off, gate, proj, w, eps, T_tokens, H, S);
+        return token_side_x8_launch<1, 256>(st, h, delta, ids, table, ld_table, off, gate, proj, w, eps, T_tokens, H, S);
     }
 #define TS_GO(T_, SB_)                                                                                         \
     hipLaunchKernelGGL((token_side_kernel<T_, SB_>), grid, block, 0, st, h, (const T_*)delta, ids, (const T_*)table, \
