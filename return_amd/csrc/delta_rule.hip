@@ -12,7 +12,7 @@
 // head of some wider rows; ag, rows [a: H*D | c: H*V], the decay's and the output gate's projections.
 //
 // Two kernels. The recurrence: a workgroup takes (head, VB columns of S, request) and walks the
-// request's rows in chunks of DR_TC; for a chunk everything that does not depend on S (decays, unit
+// request's rows in chunks of up to DR_TC_MAX; for a chunk everything that does not depend on S (decays, unit
 // vectors, beta) is prepared in LDS by all threads, then the recurrence runs over the chunk without a
 // barrier and writes the read-outs o in 32-bit. A column j of S belongs to RS neighbouring lanes, each
 // with DPT rows in registers; the two sums over rows are finished by data-parallel moves. Columns of
@@ -21,7 +21,7 @@
 // over all its columns, weighs and gates it: a wave per (row, head).
 #include "common.h"
 
-#define DR_TC 32
+#define DR_TC_MAX 32      // rows of a chunk; fewer where a head's rows would not fit the LDS
 #define DR_PAD 4
 
 __device__ __forceinline__ float dr_sigmoid(float x) { return 1.f / (1.f + expf(-x)); }
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ b, long long ld_b, const T* __restrict__ ag,
     long long ld_ag, const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ S,
     const int* __restrict__ cu_q, const int* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int D, int V,
-    int RS, int VB) {
+    int RS, int VB, int TC) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int tid = threadIdx.x, NT = blockDim.x, lane = tid & 63, wave = tid >> 6, n_waves = NT >> 6;
     const int col_blocks = (V + VB - 1) / VB;
@@ -65,10 +65,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const int PS = DPT + DR_PAD;                    // a lane group's rows in LDS, padded against bank conflicts
     const int DP = RS * PS;
     float* k_s = smem;                              // [TC][DP]
-    float* q_s = k_s + DR_TC * DP;                  // [TC][DP]
-    float* g_s = q_s + DR_TC * DP;                  // [TC][DP]
-    float* v_s = g_s + DR_TC * DP;                  // [TC][VB]
-    float* beta_s = v_s + DR_TC * VB;               // [TC]
+    float* q_s = k_s + TC * DP;                     // [TC][DP]
+    float* g_s = q_s + TC * DP;                     // [TC][DP]
+    float* v_s = g_s + TC * DP;                     // [TC][VB]
+    float* beta_s = v_s + TC * VB;                  // [TC]
 
     const int jl = tid / RS, rp = tid % RS, j = j0 + jl;
     const bool live = jl < VB && j < V;
@@ -83,8 +83,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     const float q_scale = 1.0f / sqrtf((float)D);
     const int Dfull = RS * DPT;
 
-    for (int c0 = 0; c0 < q_len; c0 += DR_TC) {
-        const int nt = min(DR_TC, q_len - c0);
+    for (int c0 = 0; c0 < q_len; c0 += TC) {
+        const int nt = min(TC, q_len - c0);
         // ---- what the chunk's rows bring, into LDS
         if (tid < nt) beta_s[tid] = dr_sigmoid(to_f(b[(size_t)(base + c0 + tid) * ld_b + h]));
         for (int idx = tid; idx < nt * VB; idx += NT) {
@@ -234,21 +234,27 @@ static bool delta_rule_plan(int D, int V, int* RS_out, int* DPT_out, int* VB_out
     return true;
 }
 
-static size_t delta_rule_lds(int DPT, int RS, int VB) {
-    return sizeof(float) * ((size_t)DR_TC * (3 * RS * (DPT + DR_PAD) + VB) + DR_TC);
+static size_t delta_rule_lds(int DPT, int RS, int VB, int TC) {
+    return sizeof(float) * ((size_t)TC * (3 * RS * (DPT + DR_PAD) + VB) + TC);
+}
+// rows of a chunk: as many as fit, a power of two from 4 to DR_TC_MAX (0: not even four)
+static int delta_rule_chunk(int DPT, int RS, int VB) {
+    for (int tc = DR_TC_MAX; tc >= 4; tc >>= 1)
+        if (delta_rule_lds(DPT, RS, VB, tc) <= 150 * 1024) return tc;
+    return 0;
 }
 
 extern "C" int ra_delta_rule_fits(int D, int V) {
     int RS, DPT, VB;
     if (!delta_rule_plan(D, V, &RS, &DPT, &VB)) return 0;
-    return delta_rule_lds(DPT, RS, VB) <= 160 * 1024 ? 1 : 0;
+    return delta_rule_chunk(DPT, RS, VB) > 0 ? 1 : 0;
 }
 
 template <typename T>
 static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, size_t lds, const void* qkv, long long ld_qkv,
                              const void* b, long long ld_b, const void* ag, long long ld_ag, const float* A_log,
                              const float* dt_bias, float* S, const int* cu_q, const int* slot_ids, float* o_raw, int H, int G,
-                             int D, int V, int RS, int VB) {
+                             int D, int V, int RS, int VB, int TC) {
 #define DR_GO(DPT_)                                                                                               \
     do {                                                                                                          \
         if (lds > 64 * 1024 &&                                                                                    \
@@ -256,7 +262,7 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
                                 (int)lds) != hipSuccess)                                                          \
             return RA_ERR_LAUNCH;                                                                                 \
         hipLaunchKernelGGL((delta_rule_kernel<T, DPT_>), grid, block, lds, st, (const T*)qkv, ld_qkv, (const T*)b, ld_b, \
-                           (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, D, V, RS, VB);       \
+                           (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, D, V, RS, VB, TC);   \
     } while (0)
     switch (DPT) {
         case 4: DR_GO(4); break;
@@ -282,8 +288,9 @@ extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, l
     if (ld_qkv < (long long)2 * G * D + (long long)H * V || ld_b < H || ld_ag < (long long)H * D + (long long)H * V)
         return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
-    const size_t lds = delta_rule_lds(DPT, RS, VB);
-    if (lds > 160 * 1024) return RA_ERR_ARG;
+    const int TC = delta_rule_chunk(DPT, RS, VB);
+    if (TC <= 0) return RA_ERR_ARG;
+    const size_t lds = delta_rule_lds(DPT, RS, VB, TC);
     const int col_blocks = (V + VB - 1) / VB;
     if ((long long)H * col_blocks > 0x7fffffffLL) return RA_ERR_ARG;
     dim3 grid(H * col_blocks, n_seqs), block(((VB * RS + 63) / 64) * 64);
@@ -291,10 +298,10 @@ extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, l
     int rc;
     if (dtype == RA_DTYPE_F32)
         rc = delta_rule_launch<float>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
-                                      slot_ids, o_raw, H, G, D, V, RS, VB);
+                                      slot_ids, o_raw, H, G, D, V, RS, VB, TC);
     else
         rc = delta_rule_launch<bf16>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
-                                     slot_ids, o_raw, H, G, D, V, RS, VB);
+                                     slot_ids, o_raw, H, G, D, V, RS, VB, TC);
     if (rc != RA_OK) return rc;
     const long long n_rows = (long long)T_tokens * H;
     dim3 ogrid((unsigned)((n_rows + 3) / 4)), oblock(256);

@@ -76,6 +76,9 @@ def build_spec(cfg: KofipelConfig) -> ModelSpec:
                                      "vocab_size": cfg.vocab, "eps": eps},
                 {"table": "side.embed", "gate": p + "side.gate", "proj": p + "side.proj", "norm": p + "side.norm"}))
         blocks.append(BlockSpec(parts, "pre_norm_conv_side"))
+    # a layer without feed-forward has no use for a second norm and convolution: a file that stores them all the same loads
+    ignorable = [f"l{i}.{name}" for i, layer in enumerate(cfg.layers) if layer.get("mlp") is None
+                 for name in ("norm2", "canon2")]
     # every run of a layer has cache layers of its own: the mixer's, then the convolutions' tails
     schedule, layer_no = [], 0
     start = int(cfg.loop["start"]) if cfg.loop else None
@@ -88,7 +91,8 @@ def build_spec(cfg: KofipelConfig) -> ModelSpec:
         architecture=cfg.architecture, hidden_size=W, vocab_size=cfg.vocab, max_position=None,
         embedding=PartSpec("token_embedding", {"vocab_size": cfg.vocab, "hidden_size": W}, {"weight": "embed"}),
         positions=positions, blocks=blocks, schedule=schedule, final_norm=norm("final.norm"),
-        head=PartSpec("linear_head", {"vocab_size": cfg.vocab, "hidden_size": W, "tied": False}, {"weight": "head"}))
+        head=PartSpec("linear_head", {"vocab_size": cfg.vocab, "hidden_size": W, "tied": False}, {"weight": "head"}),
+        ignorable=ignorable)
 
 
 register_architecture("Kofipel", KofipelConfig, build_spec)
