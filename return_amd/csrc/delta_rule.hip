@@ -72,12 +72,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
 
     const int jl = tid / RS, rp = tid % RS, j = j0 + jl;
     const bool live = jl < VB && j < V;
-    float* Sh = S + ((size_t)slot_ids[s] * H + h) * D * V;
+    // the state is kept column by column, [slot][head][V][D]: a lane's rows of its column are one run of memory,
+    // and the lanes of a wave read neighbouring runs
+    float* Sc = S + (((size_t)slot_ids[s] * H + h) * V + (live ? j : 0)) * D;
+    const bool vec = (D & 3) == 0;
     float st[DPT];
 #pragma unroll
-    for (int ii = 0; ii < DPT; ++ii) {
+    for (int ii = 0; ii < DPT; ii += 4) {
         const int i = rp * DPT + ii;
-        st[ii] = (live && i < D) ? Sh[(size_t)i * V + j] : 0.f;
+        float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            if (vec) {
+                if (i < D) v4 = *reinterpret_cast<const float4*>(Sc + i);
+            } else {
+                if (i < D) v4.x = Sc[i];
+                if (i + 1 < D) v4.y = Sc[i + 1];
+                if (i + 2 < D) v4.z = Sc[i + 2];
+                if (i + 3 < D) v4.w = Sc[i + 3];
+            }
+        }
+        st[ii] = v4.x; st[ii + 1] = v4.y; st[ii + 2] = v4.z; st[ii + 3] = v4.w;
     }
     const float neg_a = -expf(A_log[h]);
     const float q_scale = 1.0f / sqrtf((float)D);
@@ -192,9 +206,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
         __syncthreads();                                       // before the next chunk overwrites LDS
     }
 #pragma unroll
-    for (int ii = 0; ii < DPT; ++ii) {
+    for (int ii = 0; ii < DPT; ii += 4) {
         const int i = rp * DPT + ii;
-        if (live && i < D) Sh[(size_t)i * V + j] = st[ii];
+        if (!live) continue;
+        if (vec) {
+            if (i < D) *reinterpret_cast<float4*>(Sc + i) = make_float4(st[ii], st[ii + 1], st[ii + 2], st[ii + 3]);
+        } else {
+            if (i < D) Sc[i] = st[ii];
+            if (i + 1 < D) Sc[i + 1] = st[ii + 1];
+            if (i + 2 < D) Sc[i + 2] = st[ii + 2];
+            if (i + 3 < D) Sc[i + 3] = st[ii + 3];
+        }
     }
 }
 
@@ -277,19 +299,22 @@ static int delta_rule_launch(hipStream_t st, int DPT, dim3 grid, dim3 block, siz
 }
 
 // qkv [T, 2 G D + H V] rows; b: rows whose first H columns are the heads' beta (before the sigmoid); ag [T, H D + H V];
-// S fp32 [slots, H, D, V]; o_raw fp32 [T, H V] scratch; out [T, H V].
+// S fp32 [slots, H, V, D] (column by column); o_raw fp32 [T, H V] scratch; out [T, H V]; max_q_len: the longest request's rows.
 extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, long long ld_b, const void* ag,
                              long long ld_ag, const float* A_log, const float* dt_bias, const float* norm_w, float eps,
                              float* S, const int* cu_q, const int* slot_ids, float* o_raw, void* out, int n_seqs,
-                             int T_tokens, int H, int G, int D, int V, int dtype, void* stream) {
+                             int T_tokens, int max_q_len, int H, int G, int D, int V, int dtype, void* stream) {
     if (n_seqs <= 0 || T_tokens <= 0) return RA_OK;
     int RS, DPT, VB;
     if (!delta_rule_plan(D, V, &RS, &DPT, &VB) || H < 1 || G < 1 || H % G || n_seqs > 65535) return RA_ERR_ARG;
     if (ld_qkv < (long long)2 * G * D + (long long)H * V || ld_b < H || ld_ag < (long long)H * D + (long long)H * V)
         return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
-    const int TC = delta_rule_chunk(DPT, RS, VB);
-    if (TC <= 0) return RA_ERR_ARG;
+    int TC = delta_rule_chunk(DPT, RS, VB);
+    if (TC <= 0 || max_q_len < 1) return RA_ERR_ARG;
+    // no chunk longer than the step's longest request: a step of single tokens takes an eighth of the LDS, and
+    // eight times the workgroups share a CU while each waits for its state
+    while (TC > 4 && (TC >> 1) >= max_q_len) TC >>= 1;
     const size_t lds = delta_rule_lds(DPT, RS, VB, TC);
     const int col_blocks = (V + VB - 1) / VB;
     if ((long long)H * col_blocks > 0x7fffffffLL) return RA_ERR_ARG;

@@ -72,7 +72,7 @@ def _declare(lib):
         "ra_gemm_sweep_norm_bf16": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, F, I, I, P],
         "ra_causal_conv": [P, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
-        "ra_delta_rule": [P, L, P, L, P, L, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "ra_delta_rule": [P, L, P, L, P, L, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "ra_delta_rule_fits": [I, I],
         "ra_token_side": [P, P, P, P, L, I, P, P, P, F, I, I, I, I, P],
         "ra_relu_sq": [P, L, I, P],
@@ -427,7 +427,7 @@ class HipOps:
         32-bit (unit q and k, sigmoid of beta, softplus and exponentials of the decay, the norm of the read-out
         and its gate). qkv: [T, 2 G D + H V] after the short convolution; beta: [T, H] before the sigmoid;
         ag: [T, H D + H V], the decay's and the output gate's projections; each may be a column slice of wider
-        rows. state: fp32 [slots, H, D, V], updated in place; out: [T, H V]."""
+        rows. state: fp32 [slots, H, V, D] (S column by column), updated in place; out: [T, H V]."""
         ld_qkv = self._want_rows(qkv, "delta-rule q/k/v")
         ld_b = self._want_rows(beta, "delta-rule beta", qkv.dtype)
         ld_ag = self._want_rows(ag, "delta-rule decay and gate projections", qkv.dtype)
@@ -439,7 +439,7 @@ class HipOps:
             if tuple(t.shape) != shape:
                 raise KernelError(f"delta_rule: {name} is {tuple(t.shape)}, wanted {shape}")
         if qkv.shape[1] != 2 * G * D + H * V or tuple(out.shape) != (T, H * V) or tuple(beta.shape) != (T, H) \
-                or tuple(ag.shape) != (T, H * D + H * V) or T != step.n_tokens or tuple(state.shape[1:]) != (H, D, V) or H % G:
+                or tuple(ag.shape) != (T, H * D + H * V) or T != step.n_tokens or tuple(state.shape[1:]) != (H, V, D) or H % G:
             raise KernelError(f"delta_rule: qkv {tuple(qkv.shape)}, beta {tuple(beta.shape)}, ag {tuple(ag.shape)}, "
                               f"out {tuple(out.shape)}, state {tuple(state.shape)}, {H} heads over {G} of {D} x {V}, "
                               f"step of {step.n_tokens}")
@@ -450,7 +450,8 @@ class HipOps:
         o_raw = torch.empty(T, H * V, dtype=torch.float32, device=self.device)
         self._check(self.lib.ra_delta_rule(
             _ptr(qkv), ld_qkv, _ptr(beta), ld_b, _ptr(ag), ld_ag, _ptr(a_log), _ptr(dt_bias), _ptr(norm_w), float(eps),
-            _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out), step.n_seqs, T, H, G, D, V,
+            _ptr(state), _ptr(step.cu_q), _ptr(step.slot_ids), _ptr(o_raw), _ptr(out), step.n_seqs, T,
+            max(1, int(step.max_q_len)), H, G, D, V,
             _code(qkv.dtype), self._stream()), "delta_rule")
         return out
 

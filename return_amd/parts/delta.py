@@ -96,7 +96,7 @@ class ChannelDeltaMixer:
 
     def cache_spec(self):
         return StateSpec((("conv", (self.taps - 1, self.c_conv), self.rt.dtype_name),
-                          ("S", (self.H, self.D, self.V), "float32")))
+                          ("S", (self.H, self.V, self.D), "float32")))      # S column by column
 
     def forward(self, x, step, cache, write_cache=True):
         rt, ops = self.rt, self.rt.ops

@@ -132,7 +132,7 @@ def test_delta_rule_in_pieces_equals_the_plain_recurrence():
     beta = (h @ w["b"].T).float()
     ag = torch.cat([(h @ w["a1"].T) @ w["a2"].T, (h @ w["g1"].T) @ w["g2"].T], dim=1).float()
     ops = TorchOps("cpu")
-    state = torch.randn(3, H, D, V, generator=g)
+    state = torch.randn(3, H, V, D, generator=g)
     state[2].zero_()
     out = torch.empty(T, H * V)
     at = 0

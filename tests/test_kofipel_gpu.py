@@ -92,7 +92,7 @@ def test_delta_rule(ops, ref, dtype, H, G, D, V, q_lens):
     z = rnd(T, 24 + H, dtype=dtype, seed=2)
     ag = rnd(T, H * D + H * V + 8, dtype=dtype, seed=3)[:, :H * D + H * V]
     a_log, dt_bias, norm_w = rnd(H, seed=5), rnd(H * D, seed=6) - 1.0, 1 + rnd(V, seed=7, scale=0.1)
-    state_a = rnd(n + 1, H, D, V, seed=8, scale=0.3)
+    state_a = rnd(n + 1, H, V, D, seed=8, scale=0.3)
     state_b = state_a.clone()
     for round_no in range(2):                                   # the second round starts from the first's state
         step = state_step(q_lens, slots)

@@ -222,7 +222,7 @@ class TorchOps:
         gate = torch.sigmoid(ag[:, H * D:].float()).view(T, H, V)
         rep = H // G
         for s in range(step.n_seqs):
-            S = state[slots[s]]                               # [H, D, V], updated in place
+            S = state[slots[s]].transpose(1, 2)               # kept [H, V, D]; a view [H, D, V], updated in place
             for t in range(cu[s], cu[s + 1]):
                 kt, qt = k[t].repeat_interleave(rep, 0), q[t].repeat_interleave(rep, 0)    # [H, D]
                 S *= g[t][:, :, None]
