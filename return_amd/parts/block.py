@@ -136,19 +136,28 @@ class ConvSideBlock:
     def step_needs(self):
         return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
 
+    @staticmethod
+    def _normed(norm, conv, h, pending, step, tails, tail_name):
+        """What a sublayer reads: the norm of the stream (pending added first) and, if there is one, the convolution
+        behind it; in a step of single tokens both as one kernel where the kernel set has it."""
+        if conv is None:
+            return norm.forward(h, pending)
+        ops = conv.rt.ops
+        if step.all_decode and hasattr(ops, "add_rmsnorm_conv") and hasattr(norm, "weight") and hasattr(conv, "weight"):
+            out = conv.rt.empty(h.shape[0], conv.size)
+            if ops.add_rmsnorm_conv(h, pending, norm.weight, norm.eps, conv.weight, tails[tail_name], step, out):
+                return out
+        return conv.forward(norm.forward(h, pending), step, tails[tail_name])
+
     def forward(self, h, pending, step, cache, write_cache=True):
         views = () if cache is None else tuple(cache) if isinstance(cache, (tuple, list)) else (cache,)
         n = len(self._mixer_specs)
         mixer_cache = None if n == 0 else views[0] if n == 1 else views[:n]
         tails = views[n].tensors if self._tails is not None else None
-        x = self.mixer_norm.forward(h, pending)
-        if self.mixer_conv is not None:
-            x = self.mixer_conv.forward(x, step, tails["mixer_tail"])
+        x = self._normed(self.mixer_norm, self.mixer_conv, h, pending, step, tails, "mixer_tail")
         pending = self.mixer.forward(x, step, mixer_cache, write_cache)
         if self.feed_forward is not None:
-            x = self.feed_forward_norm.forward(h, pending)
-            if self.feed_forward_conv is not None:
-                x = self.feed_forward_conv.forward(x, step, tails["feed_forward_tail"])
+            x = self._normed(self.feed_forward_norm, self.feed_forward_conv, h, pending, step, tails, "feed_forward_tail")
             pending = self.feed_forward.forward(x, step)
         if self.token_input is not None:
             self.token_input.forward(h, pending, step)
