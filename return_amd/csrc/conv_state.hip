@@ -101,69 +101,3 @@ extern "C" int ra_causal_conv(const void* x, long long ld_x, const float* w, voi
                            (bf16*)tail, cu_q, slot_ids, (bf16*)out, ld_out, C, taps, flags);
     return ra_launch_status();
 }
-
-// ------------------------------------------------------------------ norm and convolution in one, for steps of single tokens
-// Every request brings one row: h += delta; n = h * rsqrt(mean(h^2) + eps) * nw, rounded to the storage type as
-// the norm kernel's result is; out = n + sum_j cw[:, j] * (tail, n)_j; the tail moves on by n. One workgroup per
-// row, a thread's columns in registers between the phases. H <= 256 * FUSE_MAX_CPT.
-#define FUSE_MAX_CPT 32
-template <typename T>
-__global__ __launch_bounds__(256) void add_rmsnorm_conv_kernel(
-    float* __restrict__ h, const T* __restrict__ delta, const float* __restrict__ nw, float eps,
-    const float* __restrict__ cw, T* __restrict__ tail, const int* __restrict__ slot_ids, T* __restrict__ out, int H,
-    int taps) {
-    __shared__ float red[16];
-    const int row = blockIdx.x, tid = threadIdx.x;
-    float* hr = h + (size_t)row * H;
-    float v[FUSE_MAX_CPT];
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < FUSE_MAX_CPT; ++i) {
-        const int c = tid + 256 * i;
-        v[i] = 0.f;
-        if (c < H) {
-            v[i] = hr[c];
-            if (delta != nullptr) {
-                v[i] += to_f(delta[(size_t)row * H + c]);
-                hr[c] = v[i];
-            }
-            ss = fmaf(v[i], v[i], ss);
-        }
-    }
-    ss = block_sum(ss, red);
-    const float rstd = 1.0f / sqrtf(ss / (float)H + eps);
-    const int back = taps - 1;
-    T* my_tail = tail + (size_t)slot_ids[row] * back * H;
-#pragma unroll
-    for (int i = 0; i < FUSE_MAX_CPT; ++i) {
-        const int c = tid + 256 * i;
-        if (c >= H) continue;
-        const float n = round_to<T>(v[i] * rstd * nw[c]);
-        float y = 0.f;
-        for (int j = 0; j < back; ++j) {
-            const float old = to_f(my_tail[(size_t)j * H + c]);
-            y = fmaf(cw[(size_t)c * taps + j], old, y);
-            if (j > 0) my_tail[(size_t)(j - 1) * H + c] = from_f<T>(old);
-        }
-        y = fmaf(cw[(size_t)c * taps + back], n, y);
-        if (back > 0) my_tail[(size_t)(back - 1) * H + c] = from_f<T>(n);
-        out[(size_t)row * H + c] = from_f<T>(n + y);
-    }
-}
-
-// h fp32 [rows, H]; delta [rows, H] or null; tail [slots, taps-1, H]; out [rows, H]; request i is row i.
-extern "C" int ra_add_rmsnorm_conv(float* h, const void* delta, const float* nw, float eps, const float* cw, void* tail,
-                                   const int* slot_ids, void* out, int rows, int H, int taps, int dtype, void* stream) {
-    if (rows <= 0) return RA_OK;
-    if (H < 1 || H > 256 * FUSE_MAX_CPT || taps < 1 || taps > CONV_MAX_TAPS) return RA_ERR_ARG;
-    dim3 grid(rows), block(256);
-    if (dtype == RA_DTYPE_F32)
-        hipLaunchKernelGGL(add_rmsnorm_conv_kernel<float>, grid, block, 0, (hipStream_t)stream, h, (const float*)delta, nw,
-                           eps, cw, (float*)tail, slot_ids, (float*)out, H, taps);
-    else if (dtype == RA_DTYPE_BF16)
-        hipLaunchKernelGGL(add_rmsnorm_conv_kernel<bf16>, grid, block, 0, (hipStream_t)stream, h, (const bf16*)delta, nw,
-                           eps, cw, (bf16*)tail, slot_ids, (bf16*)out, H, taps);
-    else
-        return RA_ERR_ARG;
-    return ra_launch_status();
-}

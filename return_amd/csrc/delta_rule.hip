@@ -11,14 +11,16 @@
 // (G heads of D for q and k, H heads of V for v; head h reads q/k head h / (H/G)); b, one column per
 // head of some wider rows; ag, rows [a: H*D | c: H*V], the decay's and the output gate's projections.
 //
-// Two kernels. The recurrence: a workgroup takes (head, VB columns of S, request) and walks the
+// The recurrence (in two forms, see below) and the output. The recurrence: a workgroup takes (head, VB columns of S, request) and walks the
 // request's rows in chunks of up to DR_TC_MAX; for a chunk everything that does not depend on S (decays, unit
 // vectors, beta) is prepared in LDS by all threads, then the recurrence runs over the chunk without a
 // barrier and writes the read-outs o in 32-bit. A column j of S belongs to RS neighbouring lanes, each
 // with DPT rows in registers; the two sums over rows are finished by data-parallel moves. Columns of
 // one head are independent, so a head is spread over V / VB workgroups: the walk over the tokens is the
 // long pole, and it is as long for 16 columns as for 128. The output kernel norms a head's read-out
-// over all its columns, weighs and gates it: a wave per (row, head).
+// over all its columns, weighs and gates it: a wave per (row, head). Steps whose longest request has eight
+// rows or more take the recurrence kernel with feeder waves (below); single tokens and short portions the plain
+// one, which needs half the threads, few registers and little LDS, so that many workgroups share a CU.
 #include "common.h"
 
 #define DR_TC_MAX 32      // rows of a chunk; fewer where a head's rows would not fit the LDS
@@ -220,6 +222,211 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) voi
     }
 }
 
+// Sum over a wave's 64 lanes, in every lane, without LDS: inside each row of 16 lanes by data-parallel moves
+// (lane ^ 1, lane ^ 2, the other quad of eight, the other half of the row), then over the four rows by lane swaps.
+__device__ __forceinline__ float dr_wave_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));
+    return rows_sum(v);
+}
+
+// Waves of two kinds. The first DR_WALKERS / 64 waves walk the tokens: column j of S belongs to RS neighbouring
+// lanes, each with DPT rows in registers. The other DR_FEEDERS / 64 waves prepare the next chunk meanwhile, into
+// the other of two LDS buffers: a feeder wave takes every other row of the chunk, asks for all its rows' q, k
+// and decay projections at once, forms the unit vectors with sums over its own lanes (no trip through LDS) and the
+// decays, and writes them where the walkers will read them. A workgroup is alone on its CU, and a chunk's loads
+// would otherwise each cost the walk a trip to memory; this way the walk never waits for memory.
+#define DR_WALKERS 128
+#define DR_FEEDERS 128
+#define DR_BATCH 32          // elements of q, k and decay projection that a feeder lane asks for at once
+template <typename T, int DPT>
+__global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_waves_per_eu(1, 2))) void delta_rule_fed_kernel(
+    const T* __restrict__ qkv, long long ld_qkv, const T* __restrict__ b, long long ld_b, const T* __restrict__ ag,
+    long long ld_ag, const float* __restrict__ A_log, const float* __restrict__ dt_bias, float* __restrict__ S,
+    const int* __restrict__ cu_q, const int* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int D, int V,
+    int RS, int VB, int TC) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int col_blocks = (V + VB - 1) / VB;
+    const int h = blockIdx.x / col_blocks, j0 = (blockIdx.x - h * col_blocks) * VB;
+    const int s = blockIdx.y, kvh = h / (H / G);
+    const int base = cu_q[s], q_len = cu_q[s + 1] - base;
+    if (q_len <= 0) return;
+    const int PS = DPT + DR_PAD;                    // a lane group's rows in LDS, padded against bank conflicts
+    const int DP = RS * PS;
+    const int BUF = (TC * (3 * DP + VB) + TC + 3) & ~3;        // floats of one buffer: k, q, g [TC][DP], v [TC][VB], beta [TC]
+    const int Dfull = RS * DPT;
+    const bool feeder = tid >= DR_WALKERS;
+    const float neg_a = -expf(A_log[h]);
+    const float q_scale = 1.0f / sqrtf((float)D);
+
+    // ---- a feeder's work for the chunk that starts at row c0, into buffer `to`
+    auto feed = [&](int c0, int to) {
+        float* k_s = smem + (size_t)to * BUF;
+        float* q_s = k_s + TC * DP;
+        float* g_s = q_s + TC * DP;
+        float* v_s = g_s + TC * DP;
+        float* beta_s = v_s + TC * VB;
+        const int ft = tid - DR_WALKERS, fw = ft >> 6;
+        const int nt = min(TC, q_len - c0);
+        constexpr int EPL = (8 * DPT + 63) / 64;            // elements of a row per lane (RS <= 8)
+        constexpr int ROWS = DR_BATCH / EPL;                // rows a wave asks for at once
+        for (int t0 = fw; t0 < nt; t0 += (DR_FEEDERS / 64) * ROWS) {
+            float fq[ROWS][EPL], fk[ROWS][EPL], fa[ROWS][EPL];
+#pragma unroll
+            for (int m = 0; m < ROWS; ++m) {
+                const int tt = t0 + m * (DR_FEEDERS / 64);
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    const int i = lane + 64 * e;
+                    fq[m][e] = fk[m][e] = fa[m][e] = 0.f;
+                    if (tt < nt && i < D) {
+                        const T* row = qkv + (size_t)(base + c0 + tt) * ld_qkv;
+                        fq[m][e] = to_f(row[kvh * D + i]);
+                        fk[m][e] = to_f(row[G * D + kvh * D + i]);
+                        fa[m][e] = to_f(ag[(size_t)(base + c0 + tt) * ld_ag + h * D + i]) + dt_bias[h * D + i];
+                    }
+                }
+            }
+            if (t0 == fw) {
+                // the chunk's values and betas: asked for behind the first batch's loads, so that all are on their way together
+                float bv = ft < nt ? to_f(b[(size_t)(base + c0 + ft) * ld_b + h]) : 0.f;
+                for (int idx0 = ft; idx0 < nt * VB; idx0 += 4 * DR_FEEDERS) {
+                    float vv[4];
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const int idx = idx0 + x * DR_FEEDERS;
+                        const int tt = idx / VB, jj = idx - tt * VB;
+                        vv[x] = (idx < nt * VB && j0 + jj < V)
+                                    ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
+                    }
+#pragma unroll
+                    for (int x = 0; x < 4; ++x)
+                        if (idx0 + x * DR_FEEDERS < nt * VB) v_s[idx0 + x * DR_FEEDERS] = vv[x];
+                }
+                if (ft < nt) beta_s[ft] = dr_sigmoid(bv);
+            }
+#pragma unroll
+            for (int m = 0; m < ROWS; ++m) {
+                const int tt = t0 + m * (DR_FEEDERS / 64);
+                if (tt >= nt) break;
+                float sk = 0.f, sq = 0.f;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    sk = fmaf(fk[m][e], fk[m][e], sk);
+                    sq = fmaf(fq[m][e], fq[m][e], sq);
+                }
+                sk = 1.0f / sqrtf(dr_wave_sum(sk) + 1e-6f);
+                sq = q_scale / sqrtf(dr_wave_sum(sq) + 1e-6f);
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) {
+                    const int i = lane + 64 * e;
+                    if (i < Dfull) {
+                        const int at = tt * DP + (i / DPT) * PS + (i % DPT);
+                        k_s[at] = fk[m][e] * sk;
+                        q_s[at] = fq[m][e] * sq;
+                        g_s[at] = i < D ? dr_decay(neg_a, fa[m][e]) : 1.f;
+                    }
+                }
+            }
+        }
+    };
+
+    // ---- a walker's state: its rows of its column, kept column by column in memory
+    const int jl = tid / RS, rp = tid % RS, j = j0 + jl;
+    const bool live = !feeder && jl < VB && j < V;
+    // the state is kept column by column, [slot][head][V][D]: a lane's rows of its column are one run of memory,
+    // and the lanes of a wave read neighbouring runs
+    float* Sc = S + (((size_t)slot_ids[s] * H + h) * V + (live ? j : 0)) * D;
+    const bool vec = (D & 3) == 0;
+    float st[DPT];
+#pragma unroll
+    for (int ii = 0; ii < DPT; ii += 4) {
+        const int i = rp * DPT + ii;
+        float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) {
+            if (vec) {
+                if (i < D) v4 = *reinterpret_cast<const float4*>(Sc + i);
+            } else {
+                if (i < D) v4.x = Sc[i];
+                if (i + 1 < D) v4.y = Sc[i + 1];
+                if (i + 2 < D) v4.z = Sc[i + 2];
+                if (i + 3 < D) v4.w = Sc[i + 3];
+            }
+        }
+        st[ii] = v4.x; st[ii + 1] = v4.y; st[ii + 2] = v4.z; st[ii + 3] = v4.w;
+    }
+
+    if (feeder) feed(0, 0);
+    __syncthreads();
+    int it = 0;
+    for (int c0 = 0; c0 < q_len; c0 += TC, ++it) {
+        const int nt = min(TC, q_len - c0);
+        const int cur = it & 1;
+        if (feeder) {
+            if (c0 + TC < q_len) feed(c0 + TC, cur ^ 1);
+        } else {
+            const float* k_s = smem + (size_t)cur * BUF;
+            const float* q_s = k_s + TC * DP;
+            const float* g_s = q_s + TC * DP;
+            const float* v_s = g_s + TC * DP;
+            const float* beta_s = v_s + TC * VB;
+            // ---- the recurrence over the chunk
+            for (int tt = 0; tt < nt; ++tt) {
+                const float* kr = k_s + tt * DP + rp * PS;
+                const float* qr = q_s + tt * DP + rp * PS;
+                const float* gr = g_s + tt * DP + rp * PS;
+                float kreg[DPT];
+                float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;     // four chains, so that no sum waits for the one before
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4*>(kr + ii);
+                    const float4 g4 = *reinterpret_cast<const float4*>(gr + ii);
+                    kreg[ii] = k4.x; kreg[ii + 1] = k4.y; kreg[ii + 2] = k4.z; kreg[ii + 3] = k4.w;
+                    st[ii] *= g4.x; st[ii + 1] *= g4.y; st[ii + 2] *= g4.z; st[ii + 3] *= g4.w;
+                    a0 = fmaf(st[ii], k4.x, a0);
+                    a1 = fmaf(st[ii + 1], k4.y, a1);
+                    a2 = fmaf(st[ii + 2], k4.z, a2);
+                    a3 = fmaf(st[ii + 3], k4.w, a3);
+                }
+                const float acc = dr_group_sum((a0 + a1) + (a2 + a3), RS);
+                const float u = beta_s[tt] * (v_s[tt * VB + (live ? jl : 0)] - acc);
+                float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii += 4) {
+                    const float4 q4 = *reinterpret_cast<const float4*>(qr + ii);
+                    st[ii] = fmaf(kreg[ii], u, st[ii]);
+                    st[ii + 1] = fmaf(kreg[ii + 1], u, st[ii + 1]);
+                    st[ii + 2] = fmaf(kreg[ii + 2], u, st[ii + 2]);
+                    st[ii + 3] = fmaf(kreg[ii + 3], u, st[ii + 3]);
+                    o0 = fmaf(st[ii], q4.x, o0);
+                    o1 = fmaf(st[ii + 1], q4.y, o1);
+                    o2 = fmaf(st[ii + 2], q4.z, o2);
+                    o3 = fmaf(st[ii + 3], q4.w, o3);
+                }
+                const float o = dr_group_sum((o0 + o1) + (o2 + o3), RS);
+                if (live && rp == 0) o_raw[(size_t)(base + c0 + tt) * H * V + h * V + j] = o;
+            }
+        }
+        __syncthreads();                                       // the next chunk is complete; this one may be overwritten
+    }
+#pragma unroll
+    for (int ii = 0; ii < DPT; ii += 4) {
+        const int i = rp * DPT + ii;
+        if (!live) continue;
+        if (vec) {
+            if (i < D) *reinterpret_cast<float4*>(Sc + i) = make_float4(st[ii], st[ii + 1], st[ii + 2], st[ii + 3]);
+        } else {
+            if (i < D) Sc[i] = st[ii];
+            if (i + 1 < D) Sc[i + 1] = st[ii + 1];
+            if (i + 2 < D) Sc[i + 2] = st[ii + 2];
+            if (i + 3 < D) Sc[i + 3] = st[ii + 3];
+        }
+    }
+}
+
 // out[t, h, :] = o[t, h, :] / sqrt(mean(o^2) + eps) * norm_w * sigmoid(c[t, h, :]): a wave per (row, head)
 template <typename T>
 __global__ __launch_bounds__(256) void delta_out_kernel(const float* __restrict__ o_raw, const T* __restrict__ gate,
@@ -266,10 +473,47 @@ static int delta_rule_chunk(int DPT, int RS, int VB) {
     return 0;
 }
 
+// The same for the kernel with feeder waves: two buffers
+static size_t delta_rule_fed_lds(int DPT, int RS, int VB, int TC) {
+    return 2 * sizeof(float) * (((size_t)TC * (3 * RS * (DPT + DR_PAD) + VB) + TC + 3) & ~(size_t)3);
+}
+static int delta_rule_fed_chunk(int DPT, int RS, int VB) {
+    for (int tc = DR_TC_MAX; tc >= 8; tc >>= 1)
+        if (delta_rule_fed_lds(DPT, RS, VB, tc) <= 150 * 1024) return tc;
+    return 0;
+}
+
 extern "C" int ra_delta_rule_fits(int D, int V) {
     int RS, DPT, VB;
     if (!delta_rule_plan(D, V, &RS, &DPT, &VB)) return 0;
     return delta_rule_chunk(DPT, RS, VB) > 0 ? 1 : 0;
+}
+
+template <typename T>
+static int delta_rule_fed_launch(hipStream_t st, int DPT, dim3 grid, size_t lds, const void* qkv, long long ld_qkv,
+                                 const void* b, long long ld_b, const void* ag, long long ld_ag, const float* A_log,
+                                 const float* dt_bias, float* S, const int* cu_q, const int* slot_ids, float* o_raw, int H,
+                                 int G, int D, int V, int RS, int VB, int TC) {
+#define DR_FED(DPT_)                                                                                                  \
+    do {                                                                                                              \
+        if (lds > 64 * 1024 &&                                                                                        \
+            hipFuncSetAttribute((const void*)delta_rule_fed_kernel<T, DPT_>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                (int)lds) != hipSuccess)                                                              \
+            return RA_ERR_LAUNCH;                                                                                     \
+        hipLaunchKernelGGL((delta_rule_fed_kernel<T, DPT_>), grid, dim3(DR_WALKERS + DR_FEEDERS), lds, st, (const T*)qkv, \
+                           ld_qkv, (const T*)b, ld_b, (const T*)ag, ld_ag, A_log, dt_bias, S, cu_q, slot_ids, o_raw, H, G, \
+                           D, V, RS, VB, TC);                                                                         \
+    } while (0)
+    switch (DPT) {
+        case 4: DR_FED(4); break;
+        case 8: DR_FED(8); break;
+        case 16: DR_FED(16); break;
+        case 32: DR_FED(32); break;
+        case 64: DR_FED(64); break;
+        default: return RA_ERR_ARG;
+    }
+#undef DR_FED
+    return ra_launch_status();
 }
 
 template <typename T>
@@ -321,7 +565,29 @@ extern "C" int ra_delta_rule(const void* qkv, long long ld_qkv, const void* b, l
     dim3 grid(H * col_blocks, n_seqs), block(((VB * RS + 63) / 64) * 64);
     hipStream_t st = (hipStream_t)stream;
     int rc;
-    if (dtype == RA_DTYPE_F32)
+    // requests of eight rows and more: the kernel whose feeder waves prepare the next chunk while this one is walked
+    // (while the workgroups are few: from about one and a half per CU on, the CUs' other workgroups fill the waits, and
+    // the plain kernel's smaller footprint wins: measured, 32 heads of 128 x 128, four requests of 512 rows 1.48 against
+    // 1.77 ms, one of 2,048 rows 2.75 against 1.76 ms)
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    const bool few = (long long)grid.x * grid.y <= (long long)cus * 3 / 2;
+    const int TCF = (max_q_len >= 8 && few) ? delta_rule_fed_chunk(DPT, RS, VB) : 0;
+    if (TCF > 0 && VB * RS <= DR_WALKERS) {
+        int tcf = TCF;
+        while (tcf > 8 && (tcf >> 1) >= max_q_len) tcf >>= 1;
+        const size_t flds = delta_rule_fed_lds(DPT, RS, VB, tcf);
+        if (dtype == RA_DTYPE_F32)
+            rc = delta_rule_fed_launch<float>(st, DPT, grid, flds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
+                                              slot_ids, o_raw, H, G, D, V, RS, VB, tcf);
+        else
+            rc = delta_rule_fed_launch<bf16>(st, DPT, grid, flds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
+                                             slot_ids, o_raw, H, G, D, V, RS, VB, tcf);
+    } else if (dtype == RA_DTYPE_F32)
         rc = delta_rule_launch<float>(st, DPT, grid, block, lds, qkv, ld_qkv, b, ld_b, ag, ld_ag, A_log, dt_bias, S, cu_q,
                                       slot_ids, o_raw, H, G, D, V, RS, VB, TC);
     else

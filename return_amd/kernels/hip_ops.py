@@ -72,7 +72,6 @@ def _declare(lib):
         "ra_gemm_sweep_norm_bf16": [P, P, P, I, I, I, I, I, I, P, I, I, F, P, P, P, P],
         "ra_attention_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P, F, I, I, P],
         "ra_causal_conv": [P, L, P, P, P, P, P, L, I, I, I, I, I, I, P],
-        "ra_add_rmsnorm_conv": [P, P, P, F, P, P, P, P, I, I, I, I, P],
         "ra_delta_rule": [P, L, P, L, P, L, P, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "ra_delta_rule_fits": [I, I],
         "ra_token_side": [P, P, P, P, L, I, P, P, P, F, I, I, I, I, P],
@@ -419,33 +418,6 @@ class HipOps:
             step.max_q_len, C, taps, (1 if add_input else 0) | (2 if silu else 0), _code(x.dtype), self._stream()),
             "causal_conv")
         return out
-
-    def add_rmsnorm_conv(self, h, delta, norm_weight, eps, conv_weight, tail, step, out):
-        """A step in which every request brings one token: h += delta, RMSNorm, and the causal convolution
-        behind it (out = n + conv(n), the tail moved on) as one kernel. Returns False, having done nothing,
-        when the step or the sizes are not such (then add_rmsnorm and causal_conv do the work)."""
-        if not step.all_decode or h.shape[1] > 8192 or isinstance(delta, (ScaledRows, Slabs)):
-            return False
-        self._want(h, "residual stream", torch.float32, 2)
-        R, H = h.shape
-        self._want(norm_weight, "norm weight", torch.float32, 1)
-        self._want(conv_weight, "conv weight", torch.float32, 2)
-        self._want(out, "output", dims=2)
-        self._want(tail, "conv tail", out.dtype, 3)
-        taps = conv_weight.shape[1]
-        if delta is not None:
-            self._want(delta, "delta", out.dtype, 2)
-        if R != step.n_seqs or tuple(out.shape) != (R, H) or norm_weight.shape[0] != H or conv_weight.shape[0] != H \
-                or tuple(tail.shape[1:]) != (taps - 1, H) or (delta is not None and tuple(delta.shape) != (R, H)) \
-                or not 1 <= taps <= 8:
-            raise KernelError(f"add_rmsnorm_conv: h {tuple(h.shape)}, out {tuple(out.shape)}, conv {tuple(conv_weight.shape)}, "
-                              f"tail {tuple(tail.shape)}, step of {step.n_seqs} requests")
-        if max(step.slot_ids_host, default=0) >= tail.shape[0]:
-            raise KernelError("add_rmsnorm_conv: a request's slot lies beyond the tail's rows")
-        self._check(self.lib.ra_add_rmsnorm_conv(_ptr(h), _ptr(delta), _ptr(norm_weight), float(eps), _ptr(conv_weight),
-                                                 _ptr(tail), _ptr(step.slot_ids), _ptr(out), R, H, taps, _code(out.dtype),
-                                                 self._stream()), "add_rmsnorm_conv")
-        return True
 
     def delta_rule_fits(self, D, V):
         return bool(self.lib.ra_delta_rule_fits(int(D), int(V)))

@@ -138,16 +138,10 @@ class ConvSideBlock:
 
     @staticmethod
     def _normed(norm, conv, h, pending, step, tails, tail_name):
-        """What a sublayer reads: the norm of the stream (pending added first) and, if there is one, the convolution
-        behind it; in a step of single tokens both as one kernel where the kernel set has it."""
-        if conv is None:
-            return norm.forward(h, pending)
-        ops = conv.rt.ops
-        if step.all_decode and hasattr(ops, "add_rmsnorm_conv") and hasattr(norm, "weight") and hasattr(conv, "weight"):
-            out = conv.rt.empty(h.shape[0], conv.size)
-            if ops.add_rmsnorm_conv(h, pending, norm.weight, norm.eps, conv.weight, tails[tail_name], step, out):
-                return out
-        return conv.forward(norm.forward(h, pending), step, tails[tail_name])
+        """What a sublayer reads: the norm of the stream (pending added first) and, if there is one, the
+        convolution behind it."""
+        x = norm.forward(h, pending)
+        return x if conv is None else conv.forward(x, step, tails[tail_name])
 
     def forward(self, h, pending, step, cache, write_cache=True):
         views = () if cache is None else tuple(cache) if isinstance(cache, (tuple, list)) else (cache,)

@@ -79,33 +79,6 @@ def test_causal_conv(ops, ref, dtype, C, taps, q_lens, flags):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,taps,n,with_delta", [(72, 2, 3, True), (256, 4, 1, False), (4096, 4, 8, True), (1000, 8, 5, True),
-                                                  (8192, 3, 2, False), (64, 1, 4, True)])
-def test_norm_and_convolution_as_one_kernel(ops, ref, dtype, H, taps, n, with_delta):
-    """Steps of single tokens: the fused kernel against the norm kernel and the convolution kernel, bit for bit,
-    over two steps (the tail of the first is the second's)."""
-    slots = torch.randperm(n + 2, generator=torch.Generator().manual_seed(n)).tolist()[:n]
-    nw, cw = 1 + rnd(H, seed=1, scale=0.1), rnd(H, taps, seed=2, scale=0.5)
-    tail_a = rnd(n + 2, taps - 1, H, dtype=dtype, seed=3)
-    tail_b = tail_a.clone()
-    h_a = rnd(n, H, seed=4)
-    h_b = h_a.clone()
-    for round_no in range(2):
-        step = state_step([1] * n, slots)
-        step.all_decode = True
-        delta = rnd(n, H, dtype=dtype, seed=5 + round_no) if with_delta else None
-        a = torch.empty(n, H, dtype=dtype, device=DEV)
-        assert ops.add_rmsnorm_conv(h_a, delta, nw, 1e-5, cw, tail_a, step, a)
-        normed = torch.empty(n, H, dtype=dtype, device=DEV)
-        ops.add_rmsnorm(h_b, delta, nw, 1e-5, normed)
-        b = torch.empty_like(normed)
-        ops.causal_conv(normed, cw, tail_b, step, b, add_input=True)
-        torch.testing.assert_close(h_a, h_b, atol=0, rtol=0)
-        torch.testing.assert_close(tail_a.float(), tail_b.float(), **tol(dtype))
-        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
-
-
-@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("H,G,D,V,q_lens", [
     (4, 2, 16, 32, [1, 1, 1]), (3, 3, 12, 20, [5, 1, 33]), (2, 1, 64, 64, [40]), (6, 2, 20, 12, [2, 17]),
     (1, 1, 64, 48, [1, 19]), (2, 2, 128, 128, [1, 70]), (2, 1, 8, 256, [3]), (2, 2, 256, 16, [1, 4]), (5, 5, 7, 3, [9]),
