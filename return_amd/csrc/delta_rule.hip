@@ -271,6 +271,25 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
         float* beta_s = v_s + TC * VB;
         const int ft = tid - DR_WALKERS, fw = ft >> 6;
         const int nt = min(TC, q_len - c0);
+        // the chunk's values and betas (every feeder thread has a share, whether or not its wave has rows)
+        auto feed_values = [&]() {
+            float bv = ft < nt ? to_f(b[(size_t)(base + c0 + ft) * ld_b + h]) : 0.f;
+            for (int idx0 = ft; idx0 < nt * VB; idx0 += 4 * DR_FEEDERS) {
+                float vv[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const int idx = idx0 + x * DR_FEEDERS;
+                    const int tt = idx / VB, jj = idx - tt * VB;
+                    vv[x] = (idx < nt * VB && j0 + jj < V)
+                                ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
+                }
+#pragma unroll
+                for (int x = 0; x < 4; ++x)
+                    if (idx0 + x * DR_FEEDERS < nt * VB) v_s[idx0 + x * DR_FEEDERS] = vv[x];
+            }
+            if (ft < nt) beta_s[ft] = dr_sigmoid(bv);
+        };
+        bool values_done = false;
         constexpr int EPL = (8 * DPT + 63) / 64;            // elements of a row per lane (RS <= 8)
         constexpr int ROWS = DR_BATCH / EPL;                // rows a wave asks for at once
         for (int t0 = fw; t0 < nt; t0 += (DR_FEEDERS / 64) * ROWS) {
@@ -290,23 +309,9 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                     }
                 }
             }
-            if (t0 == fw) {
-                // the chunk's values and betas: asked for behind the first batch's loads, so that all are on their way together
-                float bv = ft < nt ? to_f(b[(size_t)(base + c0 + ft) * ld_b + h]) : 0.f;
-                for (int idx0 = ft; idx0 < nt * VB; idx0 += 4 * DR_FEEDERS) {
-                    float vv[4];
-#pragma unroll
-                    for (int x = 0; x < 4; ++x) {
-                        const int idx = idx0 + x * DR_FEEDERS;
-                        const int tt = idx / VB, jj = idx - tt * VB;
-                        vv[x] = (idx < nt * VB && j0 + jj < V)
-                                    ? to_f(qkv[(size_t)(base + c0 + tt) * ld_qkv + 2 * G * D + h * V + j0 + jj]) : 0.f;
-                    }
-#pragma unroll
-                    for (int x = 0; x < 4; ++x)
-                        if (idx0 + x * DR_FEEDERS < nt * VB) v_s[idx0 + x * DR_FEEDERS] = vv[x];
-                }
-                if (ft < nt) beta_s[ft] = dr_sigmoid(bv);
+            if (!values_done) {
+                feed_values();                               // behind the first batch's loads: all on their way together
+                values_done = true;
             }
 #pragma unroll
             for (int m = 0; m < ROWS; ++m) {
@@ -332,6 +337,7 @@ __global__ __launch_bounds__(DR_WALKERS + DR_FEEDERS) __attribute__((amdgpu_wave
                 }
             }
         }
+        if (!values_done) feed_values();
     };
 
     // ---- a walker's state: its rows of its column, kept column by column in memory

@@ -82,7 +82,8 @@ def test_causal_conv(ops, ref, dtype, C, taps, q_lens, flags):
 @pytest.mark.parametrize("H,G,D,V,q_lens", [
     (4, 2, 16, 32, [1, 1, 1]), (3, 3, 12, 20, [5, 1, 33]), (2, 1, 64, 64, [40]), (6, 2, 20, 12, [2, 17]),
     (1, 1, 64, 48, [1, 19]), (2, 2, 128, 128, [1, 70]), (2, 1, 8, 256, [3]), (2, 2, 256, 16, [1, 4]), (5, 5, 7, 3, [9]),
-    (1, 1, 384, 40, [2, 37]), (1, 1, 512, 8, [11])])
+    (1, 1, 384, 40, [2, 37]), (1, 1, 512, 8, [11]), (2, 2, 10, 100, [1, 40]), (2, 2, 100, 3, [37, 2]), (3, 3, 10, 100, [3]),
+    (2, 2, 33, 10, [70]), (1, 1, 5, 200, [9, 1]), (1, 1, 80, 48, [33])])
 def test_delta_rule(ops, ref, dtype, H, G, D, V, q_lens):
     """Two steps in a row over slots that hold something; the inputs are column slices of wider rows."""
     n = len(q_lens)
