@@ -74,13 +74,23 @@ class PagedGroup:
         if (num_pages + 1) * page_size * spec.num_kv_heads >= 2 ** 31:
             raise ValueError(f"{num_pages} pages of {page_size} rows for {spec.num_kv_heads} kv heads: the kernels "
                              "count a layer's head rows in 32 bits")
-        self.pool = torch.zeros(len(self.layers), 2, num_pages + 1, spec.num_kv_heads, page_size,
-                                spec.head_dim, dtype=dtype, device=device)
+        if spec.value_dim is None or spec.value_dim == spec.head_dim:
+            self.pool = torch.zeros(len(self.layers), 2, num_pages + 1, spec.num_kv_heads, page_size,
+                                    spec.head_dim, dtype=dtype, device=device)
+            self.value_pool = None
+        else:
+            # values of another width than the keys: a pool each, [layer, page, kv head, row in page, width]
+            self.pool = torch.zeros(len(self.layers), num_pages + 1, spec.num_kv_heads, page_size,
+                                    spec.head_dim, dtype=dtype, device=device)
+            self.value_pool = torch.zeros(len(self.layers), num_pages + 1, spec.num_kv_heads, page_size,
+                                          spec.value_dim, dtype=dtype, device=device)
         self.spare_page = num_pages
         self.pages = FreeList(num_pages, "page")
 
     def layer_pools(self, cache_layer: int) -> Tuple[torch.Tensor, torch.Tensor]:
         i = self.local[cache_layer]
+        if self.value_pool is not None:
+            return self.pool[i], self.value_pool[i]
         return self.pool[i, 0], self.pool[i, 1]
 
 
@@ -133,6 +143,8 @@ class CacheManager:
             if isinstance(spec, PagedKVSpec):
                 if spec.window is not None and spec.window < 1:
                     raise ValueError(f"cache layer {layer}: window must be at least 1")
+                if spec.chunk is not None and spec.chunk < 1:
+                    raise ValueError(f"cache layer {layer}: chunk must be at least 1")
                 by_spec.setdefault(spec, []).append(layer)
             elif isinstance(spec, StateSpec):
                 self.state_layers[layer] = spec
@@ -171,7 +183,8 @@ class CacheManager:
         total = 0
         for spec in cache_layers.values():
             if isinstance(spec, PagedKVSpec):
-                total += 2 * pages * int(page_size) * spec.num_kv_heads * spec.head_dim * item
+                width = spec.head_dim + (spec.head_dim if spec.value_dim is None else spec.value_dim)
+                total += pages * int(page_size) * spec.num_kv_heads * width * item
             elif isinstance(spec, StateSpec):
                 for _, shape, dt in spec.tensors:
                     n = 1
@@ -237,13 +250,13 @@ class CacheManager:
         full = -(-total_tokens // P)
         out = []
         for grp in self.groups:
-            w = None if grp.spec.keep_first else grp.spec.window
-            if w is None:
+            spans = [] if grp.spec.keep_first else [s for s in (grp.spec.window, grp.spec.chunk) if s is not None]
+            if not spans:
                 out.append(full)
             else:
-                # before a step the held pages start at most P-1 rows before the window;
-                # the step then adds max_portion rows
-                out.append(min(full, -(-(w + max_portion + P - 1) // P) + 1))
+                # before a step the held pages start at most P-1 rows before the window (or the chunk's
+                # first row); the step then adds max_portion rows
+                out.append(min(full, -(-(min(spans) + max_portion + P - 1) // P) + 1))
         return out
 
     def held_pages(self, rid) -> List[int]:
@@ -375,11 +388,10 @@ class CacheManager:
             if r is None:
                 continue
             for g, grp in enumerate(self.groups):
-                w = None if grp.spec.keep_first else grp.spec.window
-                if w is None:
+                # the next query sits at position seq_len; it and every later one read keys from here on
+                first_needed = grp.spec.first_needed(r.seq_len)
+                if first_needed is None:
                     continue
-                # the next query sits at position seq_len and reads keys >= seq_len - w + 1
-                first_needed = r.seq_len - w + 1
                 drop = 0
                 while drop < len(r.pages[g]) and r.first_pos[g] + (drop + 1) * P <= first_needed:
                     drop += 1
@@ -418,7 +430,7 @@ class CacheManager:
                 assert r.first_pos[g] % P == 0
                 end = r.first_pos[g] + len(r.pages[g]) * P
                 assert r.seq_len <= end, f"{rid!r}: {r.seq_len} tokens but pages end at {end}"
-                if grp.spec.window is None or grp.spec.keep_first:
+                if grp.spec.first_needed(r.seq_len) is None:
                     assert r.first_pos[g] == 0
                     assert len(r.pages[g]) == -(-r.seq_len // P), f"{rid!r}: page count off"
         slots = [r.slot for r in self.live.values()]

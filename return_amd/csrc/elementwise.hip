@@ -65,7 +65,7 @@ extern "C" int ra_embed(const void* table, const int* ids, float* out, int T, in
 template <typename T>
 __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ delta,
                                    const float* __restrict__ w, float eps, T* __restrict__ out,
-                                   const int* __restrict__ rows, int H) {
+                                   const int* __restrict__ rows, int H, float delta_scale) {
     __shared__ float scratch[16];
     const int m = blockIdx.x;
     const size_t r = rows ? (size_t)rows[m] : (size_t)m;
@@ -75,7 +75,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
     float ss = 0.f;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = hr[c];
-        if (dr) v += to_f(dr[c]);
+        if (dr) v = fmaf(delta_scale, to_f(dr[c]), v);
         if (write_back) hr[c] = v;
         ss += v * v;
     }
@@ -84,7 +84,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
     T* o = out + (size_t)m * H;
     for (int c = threadIdx.x; c < H; c += blockDim.x) {
         float v = hr[c];                       // same thread wrote it above
-        if (dr && !write_back) v += to_f(dr[c]);
+        if (dr && !write_back) v = fmaf(delta_scale, to_f(dr[c]), v);
         o[c] = from_f<T>(v * rstd * w[c]);
     }
 }
@@ -94,7 +94,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const T* __restrict__ 
 template <typename T, int VPT>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restrict__ delta,
                                        const float* __restrict__ w, float eps, T* __restrict__ out,
-                                       const int* __restrict__ rows, int H) {
+                                       const int* __restrict__ rows, int H, float delta_scale) {
     __shared__ float scratch[16];
     const int m = blockIdx.x;
     const size_t r = rows ? (size_t)rows[m] : (size_t)m;
@@ -112,13 +112,14 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restric
             if (delta) {
                 if constexpr (sizeof(T) == 2) {
                     const uint2 d = *reinterpret_cast<const uint2*>(delta + r * H + 4 * c);
-                    v[i].x += __uint_as_float(d.x << 16);
-                    v[i].y += __uint_as_float(d.x & 0xffff0000u);
-                    v[i].z += __uint_as_float(d.y << 16);
-                    v[i].w += __uint_as_float(d.y & 0xffff0000u);
+                    v[i].x = fmaf(delta_scale, __uint_as_float(d.x << 16), v[i].x);
+                    v[i].y = fmaf(delta_scale, __uint_as_float(d.x & 0xffff0000u), v[i].y);
+                    v[i].z = fmaf(delta_scale, __uint_as_float(d.y << 16), v[i].z);
+                    v[i].w = fmaf(delta_scale, __uint_as_float(d.y & 0xffff0000u), v[i].w);
                 } else {
                     const float4 d = *reinterpret_cast<const float4*>(delta + r * H + 4 * c);
-                    v[i].x += d.x; v[i].y += d.y; v[i].z += d.z; v[i].w += d.w;
+                    v[i].x = fmaf(delta_scale, d.x, v[i].x); v[i].y = fmaf(delta_scale, d.y, v[i].y);
+                    v[i].z = fmaf(delta_scale, d.z, v[i].z); v[i].w = fmaf(delta_scale, d.w, v[i].w);
                 }
             }
             if (write_back) hr[c] = v[i];
@@ -147,8 +148,9 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ h, const T* __restric
     }
 }
 
-extern "C" int ra_add_rmsnorm(float* h, const void* delta, const float* w, float eps, void* out,
-                              const int* rows, int M, int H, int dtype, void* stream) {
+// delta_scale: the row added is h + delta_scale * delta (a product with 1 is exact, so 1 gives h + delta).
+extern "C" int ra_add_scaled_rmsnorm(float* h, const void* delta, float delta_scale, const float* w, float eps, void* out,
+                                     const int* rows, int M, int H, int dtype, void* stream) {
     if (M <= 0) return RA_OK;
     hipStream_t st = (hipStream_t)stream;
     if (H % 4 == 0 && H <= 16384) {
@@ -157,22 +159,27 @@ extern "C" int ra_add_rmsnorm(float* h, const void* delta, const float* w, float
         dim3 grid(M), block(threads);
         const bool one = nv <= threads;              // one vector per thread, else up to four
         if (dtype == RA_DTYPE_F32) {
-            if (one) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<float, 1>), grid, block, 0, st, h, (const float*)delta, w, eps, (float*)out, rows, H);
-            else hipLaunchKernelGGL((add_rmsnorm_vec_kernel<float, 4>), grid, block, 0, st, h, (const float*)delta, w, eps, (float*)out, rows, H);
+            if (one) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<float, 1>), grid, block, 0, st, h, (const float*)delta, w, eps, (float*)out, rows, H, delta_scale);
+            else hipLaunchKernelGGL((add_rmsnorm_vec_kernel<float, 4>), grid, block, 0, st, h, (const float*)delta, w, eps, (float*)out, rows, H, delta_scale);
         } else {
-            if (one) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<bf16, 1>), grid, block, 0, st, h, (const bf16*)delta, w, eps, (bf16*)out, rows, H);
-            else hipLaunchKernelGGL((add_rmsnorm_vec_kernel<bf16, 4>), grid, block, 0, st, h, (const bf16*)delta, w, eps, (bf16*)out, rows, H);
+            if (one) hipLaunchKernelGGL((add_rmsnorm_vec_kernel<bf16, 1>), grid, block, 0, st, h, (const bf16*)delta, w, eps, (bf16*)out, rows, H, delta_scale);
+            else hipLaunchKernelGGL((add_rmsnorm_vec_kernel<bf16, 4>), grid, block, 0, st, h, (const bf16*)delta, w, eps, (bf16*)out, rows, H, delta_scale);
         }
         return ra_launch_status();
     }
     dim3 grid(M), block(H >= 2048 ? 512 : 256);
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(add_rmsnorm_kernel<float>, grid, block, 0, st, h,
-                           (const float*)delta, w, eps, (float*)out, rows, H);
+                           (const float*)delta, w, eps, (float*)out, rows, H, delta_scale);
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel<bf16>, grid, block, 0, st, h,
-                           (const bf16*)delta, w, eps, (bf16*)out, rows, H);
+                           (const bf16*)delta, w, eps, (bf16*)out, rows, H, delta_scale);
     return ra_launch_status();
+}
+
+extern "C" int ra_add_rmsnorm(float* h, const void* delta, const float* w, float eps, void* out,
+                              const int* rows, int M, int H, int dtype, void* stream) {
+    return ra_add_scaled_rmsnorm(h, delta, 1.0f, w, eps, out, rows, M, H, dtype, stream);
 }
 
 // The same where the part before left its result as n_slabs 32-bit shares [n_slabs, rows of h, H] (a
@@ -869,6 +876,41 @@ extern "C" int ra_qk_prepare(const void* qk, int T_tokens, int Hq, int Hkv, int 
         hipLaunchKernelGGL(qk_prepare_kernel<bf16>, grid, block, 0, (hipStream_t)stream, (const bf16*)qk, Hq, Hkv, D,
                            bias, positions, cos_t, sin_t, R, (bf16*)q_out, (bf16*)k_pool, (bf16*)v_pool, slots, P,
                            pool_rows, n_rows);
+    else
+        return RA_ERR_ARG;
+    return ra_launch_status();
+}
+
+// ------------------------------------------------------------------ the stream beside its first value, as rows of a product
+// h (the 32-bit stream) += delta_scale * delta where a delta is given; out[t] = [h[t] | h0[t]] in the storage
+// type: the rows that a projection of the stream and of the embedding's output multiplies.
+template <typename T>
+__global__ void stream_pair_rows_kernel(float* __restrict__ h, const T* __restrict__ delta, float delta_scale,
+                                        const float* __restrict__ h0, T* __restrict__ out, int H, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const size_t t = i / H;
+    const int c = (int)(i - t * H);
+    float v = h[i];
+    if (delta != nullptr) {
+        v = fmaf(delta_scale, to_f(delta[i]), v);
+        h[i] = v;
+    }
+    out[t * 2 * H + c] = from_f<T>(v);
+    out[t * 2 * H + H + c] = from_f<T>(h0[i]);
+}
+
+extern "C" int ra_stream_pair_rows(float* h, const void* delta, float delta_scale, const float* h0, void* out,
+                                   long long rows, int H, int dtype, void* stream) {
+    const long long total = rows * H;
+    if (total <= 0) return RA_OK;
+    dim3 block(256), grid((unsigned)((total + 255) / 256));
+    if (dtype == RA_DTYPE_F32)
+        hipLaunchKernelGGL(stream_pair_rows_kernel<float>, grid, block, 0, (hipStream_t)stream, h, (const float*)delta,
+                           delta_scale, h0, (float*)out, H, (size_t)total);
+    else if (dtype == RA_DTYPE_BF16)
+        hipLaunchKernelGGL(stream_pair_rows_kernel<bf16>, grid, block, 0, (hipStream_t)stream, h, (const bf16*)delta,
+                           delta_scale, h0, (bf16*)out, H, (size_t)total);
     else
         return RA_ERR_ARG;
     return ra_launch_status();

@@ -52,6 +52,16 @@ def _declare(lib):
     sigs = {
         "ra_embed": [P, P, P, I, I, I, I, P],
         "ra_add_rmsnorm": [P, P, P, F, P, P, I, I, I, P],
+        "ra_add_scaled_rmsnorm": [P, P, F, P, F, P, P, I, I, I, P],
+        "ra_stream_pair_rows": [P, P, F, P, P, L, I, I, P],
+        "ra_maps_qkv_prepare": [P, I, I, I, I, I, I, P, P, P, I, I, P, P, P, P, I, I, P],
+        "ra_attention_diff_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, F, F, F, I, P],
+        "ra_attention_diff_plain_fits": [I, I],
+        "ra_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
+        "ra_moe_plan": [P, I, I, I, P, P, P, P],
+        "ra_moe_tile_rows": [I, I, I, I],
+        "ra_moe_product": [P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "ra_moe_combine": [P, P, P, I, I, I, I, P],
         "ra_add_slabs_rmsnorm": [P, P, I, L, P, F, P, P, I, I, I, P],
         "ra_residual_add": [P, P, L, I, P],
         "ra_head_rmsnorm": [P, P, F, L, I, I, P],
@@ -223,7 +233,8 @@ class HipOps:
         self._check(self.lib.ra_embed(_ptr(table), _ptr(ids), _ptr(out), T, H, table.shape[0],
                                       _code(table.dtype), self._stream()), "embed")
 
-    def add_rmsnorm(self, h, delta, weight, eps, out, rows=None):
+    def add_rmsnorm(self, h, delta, weight, eps, out, rows=None, delta_scale=1.0):
+        """h += delta_scale * delta (in place, unless a row list is given); out = norm(h) * weight."""
         self._want(h, "residual stream", torch.float32, 2)
         self._want(weight, "norm weight", torch.float32, 1)
         self._want(out, "norm output", dims=2)
@@ -234,6 +245,8 @@ class HipOps:
             self._want(delta.tensor, "shares of the product", torch.float32, 3)
             if tuple(delta.tensor.shape[1:]) != (R, H):
                 raise KernelError(f"add_rmsnorm: shares {tuple(delta.tensor.shape)} do not match h {tuple(h.shape)}")
+            if float(delta_scale) != 1.0:
+                raise KernelError("add_rmsnorm: shares of a product are added as they are, not times a factor")
             if rows is not None:
                 self._want(rows, "row list", torch.int32, 1)
             M = R if rows is None else rows.shape[0]
@@ -254,17 +267,40 @@ class HipOps:
             M = R
         if out.shape[0] != M:
             raise KernelError(f"add_rmsnorm: out has {out.shape[0]} rows, {M} wanted")
+        if float(delta_scale) != 1.0:
+            self._check(self.lib.ra_add_scaled_rmsnorm(_ptr(h), _ptr(delta), float(delta_scale), _ptr(weight), float(eps),
+                                                       _ptr(out), _ptr(rows), M, H, _code(out.dtype), self._stream()),
+                        "add_scaled_rmsnorm")
+            return
         self._check(self.lib.ra_add_rmsnorm(_ptr(h), _ptr(delta), _ptr(weight), float(eps), _ptr(out),
                                             _ptr(rows), M, H, _code(out.dtype), self._stream()),
                     "add_rmsnorm")
 
-    def residual_add(self, h, delta):
+    def residual_add(self, h, delta, scale=1.0):
         self._want(h, "residual stream", torch.float32)
         self._want(delta, "delta")
         if h.shape != delta.shape:
             raise KernelError(f"residual_add: {tuple(h.shape)} += {tuple(delta.shape)}")
+        if float(scale) != 1.0:
+            h.add_(delta, alpha=float(scale))            # (32-bit: the sum is formed in h's type)
+            return
         self._check(self.lib.ra_residual_add(_ptr(h), _ptr(delta), h.numel(), _code(delta.dtype),
                                              self._stream()), "residual_add")
+
+    def stream_pair_rows(self, h, delta, delta_scale, h0, out):
+        """h += delta_scale * delta (delta may be None); out [T, 2H] = [h | h0] in out's type."""
+        self._want(h, "residual stream", torch.float32, 2)
+        self._want(h0, "first stream", torch.float32, 2)
+        self._want(out, "rows", dims=2)
+        T, H = h.shape
+        if h0.shape != h.shape or tuple(out.shape) != (T, 2 * H):
+            raise KernelError(f"stream_pair_rows: h {tuple(h.shape)}, h0 {tuple(h0.shape)}, out {tuple(out.shape)}")
+        if delta is not None:
+            self._want(delta, "delta", out.dtype, 2)
+            if delta.shape != h.shape:
+                raise KernelError(f"stream_pair_rows: delta {tuple(delta.shape)} does not match h {tuple(h.shape)}")
+        self._check(self.lib.ra_stream_pair_rows(_ptr(h), _ptr(delta), float(delta_scale), _ptr(h0), _ptr(out), T, H,
+                                                 _code(out.dtype), self._stream()), "stream_pair_rows")
 
     def head_rmsnorm(self, x, weight, eps):
         self._want(x, "heads", dims=3)
@@ -1140,6 +1176,151 @@ class HipOps:
         ends = [s + min(off + rows, q) for q, s in zip(step.q_lens, step.q_starts) if q != 1
                 for off in range(0, q, rows)]
         return 2 if max(ends) * len(ends) >= 1.4 * sum(ends) else 1
+
+    # ------------------------------------------------------------------ differential attention
+    def check_attention_diff_sizes(self, n_q, n_kv, D, Dv, dtype):
+        """Raises for sizes that no differential attention kernel here takes (asked when a model is built)."""
+        if n_kv < 1 or n_q % n_kv or n_q > 65535:
+            raise KernelError(f"differential attention: {n_q} query heads over {n_kv} kv heads")
+        if not self.lib.ra_attention_diff_plain_fits(int(D), int(Dv)):
+            raise KernelError(f"differential attention: maps of {D} with values of {Dv} are beyond the kernels")
+        _code(dtype)
+
+    def _pools_two_widths(self, k_pool, v_pool, n_kv, Dk, Dv, dtype):
+        for t, name, width in ((k_pool, "k pool", Dk), (v_pool, "v pool", Dv)):
+            self._want(t, name, dtype, 4)
+            if t.shape[1] != n_kv or t.shape[3] != width:
+                raise KernelError(f"{name} {tuple(t.shape)} does not hold {n_kv} heads of {width}")
+        if k_pool.shape[:3] != v_pool.shape[:3]:
+            raise KernelError("k pool and v pool differ in pages, heads or rows")
+        if k_pool.shape[0] * k_pool.shape[1] * k_pool.shape[2] >= 2 ** 31:
+            raise KernelError(f"k pool {tuple(k_pool.shape)}: the kernels count head rows in 32 bits")
+        return k_pool.shape[0] * k_pool.shape[2]
+
+    def maps_qkv_prepare(self, qkv, n_q, n_kv, maps, D, Dv, positions, cos, sin, rotary_dim, interleaved, q_out,
+                         k_pool, v_pool, slot_mapping):
+        """q/k/v preparation of an attention with several score maps per head: rows of qkv are
+        [n_q * maps * D | n_kv * maps * D | n_kv * Dv]; the first rotary_dim elements of every map of q and k are
+        rotated (pairs 2i, 2i + 1 when interleaved, else i, i + rotary_dim / 2); q to q_out [T, n_q, maps * D],
+        k and v to the rows of the pools that slot_mapping names (pools None: nothing is written)."""
+        self._want(qkv, "qkv", dims=2)
+        self._want(q_out, "q", qkv.dtype, 3)
+        self._want(positions, "positions", torch.int32, 1)
+        T, R = qkv.shape[0], int(rotary_dim)
+        if qkv.shape[1] != (n_q + n_kv) * maps * D + n_kv * Dv or tuple(q_out.shape) != (T, n_q, maps * D) \
+                or positions.shape[0] != T:
+            raise KernelError(f"maps_qkv_prepare: qkv {tuple(qkv.shape)}, q {tuple(q_out.shape)}, {T} tokens")
+        if R:
+            self._want(cos, "cos table", torch.float32, 2)
+            self._want(sin, "sin table", torch.float32, 2)
+            if R % 2 or R > D or cos.shape[1] != R // 2 or sin.shape != cos.shape:
+                raise KernelError(f"maps_qkv_prepare: rotary_dim {R}, tables {tuple(cos.shape)}, map size {D}")
+        P = 1
+        if k_pool is not None:
+            self._want(slot_mapping, "slot mapping", torch.int32, 1)
+            if slot_mapping.shape[0] != T:
+                raise KernelError("maps_qkv_prepare: slot mapping does not match the token count")
+            self._pools_two_widths(k_pool, v_pool, n_kv, maps * D, Dv, qkv.dtype)
+            P = k_pool.shape[2]
+        self._check(self.lib.ra_maps_qkv_prepare(
+            _ptr(qkv), T, n_q, n_kv, maps, D, Dv, _ptr(positions), _ptr(cos) if R else None, _ptr(sin) if R else None,
+            R, 1 if interleaved else 0, _ptr(q_out), _ptr(k_pool), _ptr(v_pool),
+            _ptr(slot_mapping) if k_pool is not None else None, P, _code(qkv.dtype), self._stream()), "maps_qkv_prepare")
+
+    def diff_prefill_tile_rows(self, D, Dv, dtype):
+        """Rows per q tile of the lists that attention_diff reads from step.prefill_tiles, or None where the
+        kernel that serves these sizes takes no list."""
+        return None
+
+    def attention_diff(self, q, out, k_pool, v_pool, step, group, scale, lam, eps, out_scale, window=0, chunk=0):
+        """Differential attention of the step's queries over the paged cache: q [T, n_q, 2 D] (two maps a head),
+        key pool rows [2 D], value pool rows [Dv], out [T, n_q, Dv] = norm(a1 - lam a2) * out_scale."""
+        self._want(q, "q", dims=3)
+        self._want(out, "attention output", q.dtype, 3)
+        T, n_q, D2 = q.shape
+        Dv = out.shape[2]
+        g = step.groups[group]
+        n_kv = k_pool.shape[1]
+        if D2 % 2 or tuple(out.shape[:2]) != (T, n_q) or T != step.n_tokens:
+            raise KernelError(f"attention_diff: q {tuple(q.shape)}, out {tuple(out.shape)}, step of {step.n_tokens}")
+        self._pools_two_widths(k_pool, v_pool, n_kv, D2, Dv, q.dtype)
+        self.check_attention_diff_sizes(n_q, n_kv, D2 // 2, Dv, q.dtype)
+        P = k_pool.shape[2]
+        tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
+        self._check(self.lib.ra_attention_diff_plain(
+            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, None, step.n_seqs, T, n_q, n_kv, D2 // 2, Dv, P,
+            float(scale), int(window), int(chunk), float(lam), float(eps), float(out_scale), _code(q.dtype),
+            self._stream()), "attention_diff_plain")
+
+    # ------------------------------------------------------------------ routed experts
+    MAX_EXPERTS = 1024
+
+    def check_moe_sizes(self, experts, top, groups, keep):
+        if not 1 <= experts <= self.MAX_EXPERTS or not 1 <= top <= min(64, experts) or groups < 1 or experts % groups \
+                or not 1 <= keep <= groups or keep * (experts // groups) < top:
+            raise KernelError(f"routed experts: {experts} experts, top {top}, {groups} groups of which {keep} stay "
+                              f"are beyond the kernels (at most {self.MAX_EXPERTS} experts, top 64)")
+
+    def moe_route(self, z, bias, top, groups, keep, norm_eps):
+        """Router logits z [T, E] (32-bit) -> (ids int32 [T, top], weights fp32 [T, top])."""
+        self._want(z, "router logits", torch.float32, 2)
+        T, E = z.shape
+        self.check_moe_sizes(E, top, groups, keep)
+        if bias is not None:
+            self._want(bias, "router correction", torch.float32, 1)
+            if bias.shape[0] != E:
+                raise KernelError(f"moe_route: correction {tuple(bias.shape)} for {E} experts")
+        ids = torch.empty(T, top, dtype=torch.int32, device=self.device)
+        weights = torch.empty(T, top, dtype=torch.float32, device=self.device)
+        self._check(self.lib.ra_moe_route(_ptr(z), _ptr(bias), T, E, int(top), int(groups), int(keep), float(norm_eps),
+                                          _ptr(ids), _ptr(weights), self._stream()), "moe_route")
+        return ids, weights
+
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down):
+        """sum_k weights[t, k] * down_e(silu(gate_e x_t) * up_e x_t), e = ids[t, k]; w_gate_up [E, 2I, H] (gate
+        rows first), w_down [E, H, I]. The pairs are grouped by expert on the device."""
+        self._want(x, "rows", dims=2)
+        self._want(ids, "expert ids", torch.int32, 2)
+        self._want(weights, "expert weights", torch.float32, 2)
+        self._want(w_gate_up, "gate-up matrices", x.dtype, 3)
+        self._want(w_down, "down matrices", x.dtype, 3)
+        T, H = x.shape
+        E, I2, _ = w_gate_up.shape
+        top, I = ids.shape[1], I2 // 2
+        if tuple(ids.shape) != (T, top) or weights.shape != ids.shape or w_gate_up.shape[2] != H or I2 % 2 \
+                or tuple(w_down.shape) != (E, H, I):
+            raise KernelError(f"moe_experts: x {tuple(x.shape)}, ids {tuple(ids.shape)}, gate-up {tuple(w_gate_up.shape)}, "
+                              f"down {tuple(w_down.shape)}")
+        n_pairs, code = T * top, _code(x.dtype)
+        out = torch.empty(T, H, dtype=x.dtype, device=self.device)
+        if n_pairs == 0:
+            return out
+        act = torch.empty(n_pairs, I, dtype=x.dtype, device=self.device)
+        y = torch.empty(n_pairs, H, dtype=x.dtype, device=self.device)
+
+        def plan(rows):
+            # (every expert may end in a tile that is not full)
+            max_tiles = min(n_pairs, n_pairs // rows + E)
+            order = torch.empty(n_pairs, dtype=torch.int32, device=self.device)
+            tiles = torch.empty(max_tiles, 3, dtype=torch.int32, device=self.device)
+            meta = torch.empty(1, dtype=torch.int32, device=self.device)
+            self._check(self.lib.ra_moe_plan(_ptr(ids), n_pairs, E, rows, _ptr(order), _ptr(tiles), _ptr(meta),
+                                             self._stream()), "moe_plan")
+            return order, tiles, meta, max_tiles, rows
+
+        # the two products may take tiles of different heights (their K differ): a plan each where they do
+        rows_up, rows_down = (int(self.lib.ra_moe_tile_rows(n_pairs, E, K, code)) for K in (H, I))
+        up = plan(rows_up)
+        down = up if rows_down == rows_up else plan(rows_down)
+        order, tiles, meta, max_tiles, rows = up
+        self._check(self.lib.ra_moe_product(_ptr(x), _ptr(w_gate_up), _ptr(act), _ptr(order), _ptr(tiles), _ptr(meta),
+                                            max_tiles, rows, I, H, top, 1, code, self._stream()), "moe_product (gate-up)")
+        order, tiles, meta, max_tiles, rows = down
+        self._check(self.lib.ra_moe_product(_ptr(act), _ptr(w_down), _ptr(y), _ptr(order), _ptr(tiles), _ptr(meta),
+                                            max_tiles, rows, H, I, 1, 0, code, self._stream()), "moe_product (down)")
+        self._check(self.lib.ra_moe_combine(_ptr(y), _ptr(weights), _ptr(out), T, top, H, code, self._stream()),
+                    "moe_combine")
+        return out
 
     # ------------------------------------------------------------------ measurement
     def stream_read(self, t, workgroups=0):

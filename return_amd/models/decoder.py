@@ -12,6 +12,7 @@ import torch
 
 from ..parts.block import BLOCKS
 from ..parts.registry import part_class
+from ..parts.runtime import unscaled
 from ..parts.spec import ModelSpec
 
 
@@ -36,6 +37,9 @@ class Decoder:
                 category, ps = b.parts[name]
                 return build(category, ps, self.positions)
             self.blocks.append(BLOCKS[b.arrangement](b, build_named))
+        self.pass_input = build("pass_input", spec.pass_input) if spec.pass_input is not None else None
+        if self.pass_input is None and any(call.pass_input is not None for call in spec.schedule):
+            raise ValueError("the run order names passes that begin with a pass input, but the model has no such part")
         self.final_norm = build("norm", spec.final_norm)
         self.head = build("head", spec.head)
         self.schedule = list(spec.schedule)
@@ -98,11 +102,17 @@ class Decoder:
         """Run the step's tokens through every call of the run order; logits [m, V] fp32 at step.logit_rows."""
         h = self.embedding.forward(step.token_ids, step)
         pending = None
-        h_in = h.clone() if any(call.add_input for call in self.schedule) else None
+        h_in = h.clone() if any(call.add_input or call.pass_input is not None for call in self.schedule) else None
         for i, call in enumerate(self.schedule):
+            if call.pass_input is not None:
+                h, pending = self.pass_input.forward(h, pending, h_in, call.pass_input)
             if call.add_input:
                 if pending is not None:                   # what the part before left goes into the stream first
-                    self.rt.ops.residual_add(h, pending)
+                    delta, factor = unscaled(pending)
+                    if factor != 1.0:
+                        self.rt.ops.residual_add(h, delta, scale=factor)
+                    else:
+                        self.rt.ops.residual_add(h, pending)
                     pending = None
                 self.rt.ops.residual_add(h, h_in)
             view = None

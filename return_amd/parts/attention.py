@@ -167,3 +167,86 @@ class PagedAttention:
 
 
 register_part("mixer", "attention", PagedAttention)
+
+
+class DifferentialAttention:
+    """Grouped-query attention with two score maps per head over the same values.
+
+    q has Hq heads of two maps [map 1 | map 2] of size D each, k has Hkv heads of the same two maps, v has
+    Hkv heads of size Dv. Each map is a softmax attention of its own (score q_m . k_m * scale over the
+    keys the mask leaves), a1 and a2; with one number for the layer,
+        lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + lambda_init,
+    the head gives  o = a1 - lambda a2,  o <- o / sqrt(mean(o^2) + eps) * (1 - lambda_init)  (the norm over the
+    head's Dv values, no weight), and the heads side by side go through the output projection.
+    Parameters: hidden_size, num_heads, num_kv_heads, head_dim (D, of one map), value_dim, scale,
+    lambda_init, eps, position (a rotary encoding of the model's, applied to each map of q and k; None:
+    none), chunk (c: position i reads j <= i with floor(i / c) = floor(j / c); None: all j <= i), window
+    (None: none). The cache keeps both maps of a token's key in one row (2 D) and the value in a row of Dv.
+    """
+
+    @staticmethod
+    def tensor_shapes(params):
+        H, Hq, Hkv, D, Dv = (params["hidden_size"], params["num_heads"], params["num_kv_heads"],
+                             params["head_dim"], params["value_dim"])
+        return {"q_proj": (Hq * 2 * D, H), "k_proj": (Hkv * 2 * D, H), "v_proj": (Hkv * Dv, H),
+                "o_proj": (H, Hq * Dv), "lq1": (D,), "lk1": (D,), "lq2": (D,), "lk2": (D,)}
+
+    @staticmethod
+    def random_init(params, role):
+        if role in ("lq1", "lk1", "lq2", "lk2"):
+            # small vectors: lambda stays near lambda_init
+            return lambda shape, gen: 0.1 * torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.hidden = int(params["hidden_size"])
+        self.n_q, self.n_kv = int(params["num_heads"]), int(params["num_kv_heads"])
+        self.d, self.dv = int(params["head_dim"]), int(params["value_dim"])
+        if self.n_q % self.n_kv:
+            raise ValueError(f"{self.n_q} query heads are not a multiple of {self.n_kv} kv heads")
+        self.scale = float(params["scale"]) if params.get("scale") is not None else self.d ** -0.5
+        self.lambda_init = float(params["lambda_init"])
+        self.eps = float(params["eps"])
+        self.chunk = int(params["chunk"]) if params.get("chunk") else None
+        self.window = int(params["window"]) if params.get("window") else None
+        self.position = (shared or {}).get(params["position"]) if params.get("position") else None
+        if params.get("position") and self.position is None:
+            raise KeyError(f"attention names position encoding {params['position']!r}, which the model lacks")
+        if self.position is not None and not hasattr(self.position, "tables"):
+            raise ValueError("differential attention rotates by tables only")
+        if hasattr(rt.ops, "check_attention_diff_sizes"):
+            rt.ops.check_attention_diff_sizes(self.n_q, self.n_kv, self.d, self.dv, rt.dtype)
+        dot = lambda a, b: float((tensors[a].double() * tensors[b].double()).sum())
+        import math
+        self.lam = math.exp(dot("lq1", "lk1")) - math.exp(dot("lq2", "lk2")) + self.lambda_init
+        self.w_qkv = rt.product(torch.cat([rt.matrix(tensors[n]) for n in ("q_proj", "k_proj", "v_proj")],
+                                          dim=0).contiguous())
+        self.w_o = rt.product(rt.matrix(tensors["o_proj"]))
+
+    def cache_spec(self):
+        return PagedKVSpec(self.n_kv, 2 * self.d, self.window, 0, self.dv, self.chunk)
+
+    def step_needs(self):
+        ops = self.rt.ops
+        rows = ops.diff_prefill_tile_rows(self.d, self.dv, self.rt.dtype) if hasattr(ops, "diff_prefill_tile_rows") else None
+        return {"prefill_tile_rows": set(rows)} if rows else {}
+
+    def forward(self, x, step, cache, write_cache=True):
+        rt, ops = self.rt, self.rt.ops
+        T, Hq, Hkv, D, Dv = x.shape[0], self.n_q, self.n_kv, self.d, self.dv
+        tables = step.groups[cache.group]
+        qkv = ops.linear(x, self.w_qkv)                              # [T, (Hq + Hkv) * 2D + Hkv * Dv]
+        cos, sin, rot = self.position.tables() if self.position is not None else (None, None, 0)
+        interleaved = getattr(self.position, "pairing", "half") == "interleaved"
+        q = rt.empty(T, Hq, 2 * D)
+        ops.maps_qkv_prepare(qkv, Hq, Hkv, 2, D, Dv, step.positions, cos, sin, rot, interleaved, q,
+                             cache.k_pool if write_cache else None, cache.v_pool if write_cache else None,
+                             tables.slot_mapping)
+        o = rt.empty(T, Hq, Dv)
+        ops.attention_diff(q, o, cache.k_pool, cache.v_pool, step, cache.group, self.scale, self.lam, self.eps,
+                           1.0 - self.lambda_init, window=self.window or 0, chunk=self.chunk or 0)
+        return ops.linear(o.view(T, Hq * Dv), self.w_o)
+
+
+register_part("mixer", "differential_attention", DifferentialAttention)

@@ -20,7 +20,7 @@ from __future__ import annotations
 
 import inspect
 
-from .runtime import NormSink, ResidualSink
+from .runtime import NormSink, ResidualSink, Scaled
 
 
 _TAKES_SINK = {}
@@ -159,7 +159,41 @@ class ConvSideBlock:
         return h, pending
 
 
-BLOCKS = {"pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock}
+class ScaledPreNormBlock:
+    """Pre-norm layer whose sublayers enter the stream times a factor m, the feed-forward optional:
+
+        h += m * mixer(mixer_norm(h));  h += m * feed_forward(feed_forward_norm(h))
+
+    Parts by name: mixer_norm, mixer and, both or neither, feed_forward_norm + feed_forward. The factor is
+    the BlockSpec's part "residual" (category "norm", kind "factor": a constant, no tensors) or 1. A
+    sublayer's output is handed on as Scaled rows, which whatever adds it into the stream multiplies."""
+
+    def __init__(self, spec, build):
+        self.mixer_norm = build("mixer_norm")
+        self.mixer = build("mixer")
+        self.feed_forward = build("feed_forward") if "feed_forward" in spec.parts else None
+        self.feed_forward_norm = build("feed_forward_norm") if self.feed_forward is not None else None
+        self.factor = float(build("residual").factor) if "residual" in spec.parts else 1.0
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def step_needs(self):
+        return self.mixer.step_needs() if hasattr(self.mixer, "step_needs") else {}
+
+    def _out(self, y):
+        return y if self.factor == 1.0 else Scaled(y, self.factor)
+
+    def forward(self, h, pending, step, cache, write_cache=True):
+        x = self.mixer_norm.forward(h, pending)
+        pending = self._out(self.mixer.forward(x, step, cache, write_cache))
+        if self.feed_forward is not None:
+            x = self.feed_forward_norm.forward(h, pending)
+            pending = self._out(self.feed_forward.forward(x, step))
+        return h, pending
+
+
+BLOCKS = {"pre_norm": PreNormBlock, "pre_norm_conv_side": ConvSideBlock, "pre_norm_scaled": ScaledPreNormBlock}
 
 
 def register_arrangement(name, cls):

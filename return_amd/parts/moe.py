@@ -1,0 +1,76 @@
+"""Routed feed-forward: a mixture of small gated feed-forward layers, of which each token uses a few.
+
+Expert e: down_e(silu(gate_e x) * (up_e x)), no biases. Router: z = W_r x in 32-bit, s = sigmoid(z);
+the choice is made on s + correction (a stored vector, one entry per expert), the weights use s alone.
+Experts form ``groups`` equal groups of neighbours; a group's score is the sum of its two largest
+choice scores, and only experts of the ``keep`` best groups can be chosen (groups 1: no such limit).
+The ``top`` eligible experts with the largest choice scores are taken; their weights are their s
+divided by the sum of those s (+ norm_eps); the output is the weighted sum of their outputs.
+
+The experts' matrices are kept stacked ([E, 2 I, H] with gate rows first, [E, H, I]); a step's (token,
+choice) pairs are grouped by expert on the device and the products run over those groups, so nothing
+of a step's routing comes back to the host.
+"""
+from __future__ import annotations
+
+import torch
+
+from .registry import register_part
+
+
+class GroupedRoutedExperts:
+    @staticmethod
+    def tensor_shapes(params):
+        H, I, E = params["hidden_size"], params["expert_size"], params["experts"]
+        shapes = {"router": (E, H), "correction": (E,)}
+        for e in range(E):
+            shapes[f"gate_{e}"] = (I, H)
+            shapes[f"up_{e}"] = (I, H)
+            shapes[f"down_{e}"] = (H, I)
+        return shapes
+
+    @staticmethod
+    def tensor_names(prefix, experts):
+        """role -> tensor name for experts stored as <prefix>e<i>.gate / .up / .down beside <prefix>router
+        and <prefix>correction."""
+        names = {"router": prefix + "router", "correction": prefix + "correction"}
+        for e in range(experts):
+            for role in ("gate", "up", "down"):
+                names[f"{role}_{e}"] = f"{prefix}e{e}.{role}"
+        return names
+
+    @staticmethod
+    def random_init(params, role):
+        if role == "correction":
+            return lambda shape, gen: 0.05 * torch.randn(*shape, generator=gen, dtype=torch.float32, device=gen.device)
+        if role == "router":
+            # logits of order one, so that the choice differs from token to token
+            return lambda shape, gen: torch.randn(*shape, generator=gen, dtype=torch.float32,
+                                                  device=gen.device) * (2.0 / params["hidden_size"] ** 0.5)
+        return "matrix"
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.rt = rt
+        self.hidden, self.inter = int(params["hidden_size"]), int(params["expert_size"])
+        self.experts, self.top = int(params["experts"]), int(params["top"])
+        self.groups, self.keep = int(params.get("groups") or 1), int(params.get("keep") or params.get("groups") or 1)
+        self.norm_eps = float(params.get("norm_eps", 1e-20))
+        E = self.experts
+        if E % self.groups or not 1 <= self.keep <= self.groups or not 1 <= self.top <= self.keep * (E // self.groups):
+            raise ValueError(f"routed experts: {E} experts in {self.groups} groups, {self.keep} kept, top {self.top}")
+        if hasattr(rt.ops, "check_moe_sizes"):
+            rt.ops.check_moe_sizes(E, self.top, self.groups, self.keep)
+        self.w_router = rt.product(rt.matrix(tensors["router"]), out_dtype=torch.float32)
+        self.correction = rt.vector32(tensors["correction"])
+        self.w_gate_up = torch.stack([torch.cat([rt.matrix(tensors[f"gate_{e}"]), rt.matrix(tensors[f"up_{e}"])], dim=0)
+                                      for e in range(E)]).contiguous()                  # [E, 2I, H]
+        self.w_down = torch.stack([rt.matrix(tensors[f"down_{e}"]) for e in range(E)]).contiguous()   # [E, H, I]
+
+    def forward(self, x, step=None):
+        ops = self.rt.ops
+        z = ops.linear(x, self.w_router, out_dtype=torch.float32)                        # [T, E]
+        ids, weights = ops.moe_route(z, self.correction, self.top, self.groups, self.keep, self.norm_eps)
+        return ops.moe_experts(x, ids, weights, self.w_gate_up, self.w_down)
+
+
+register_part("feed_forward", "grouped_routed_experts", GroupedRoutedExperts)

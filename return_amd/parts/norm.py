@@ -7,7 +7,7 @@ offset 0.0 (rollout/monkey_patch/qwen3.py:15-17).
 from __future__ import annotations
 
 from .registry import register_part
-from .runtime import ScaledRows
+from .runtime import ScaledRows, unscaled
 
 
 class RMSNorm:
@@ -39,8 +39,25 @@ class RMSNorm:
             return delta
         rows = h.shape[0] if out_rows is None else out_rows.shape[0]
         out = self.rt.empty(rows, self.size)
-        self.rt.ops.add_rmsnorm(h, delta, self.weight, self.eps, out, out_rows)
+        delta, factor = unscaled(delta)
+        if factor != 1.0:
+            self.rt.ops.add_rmsnorm(h, delta, self.weight, self.eps, out, out_rows, delta_scale=factor)
+        else:
+            self.rt.ops.add_rmsnorm(h, delta, self.weight, self.eps, out, out_rows)
         return out
 
 
+class Factor:
+    """A constant that an arrangement multiplies a sublayer's output by before it enters the stream
+    (params["factor"]); it has no tensors."""
+
+    @staticmethod
+    def tensor_shapes(params):
+        return {}
+
+    def __init__(self, params, tensors, rt, shared=None):
+        self.factor = float(params["factor"])
+
+
 register_part("norm", "rms_norm", RMSNorm)
+register_part("norm", "factor", Factor)

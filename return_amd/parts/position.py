@@ -1,4 +1,4 @@
-"""Rotary position encoding, half-split pairing.
+"""Rotary position encoding, half-split pairing (or, with pairing "interleaved", element 2i with 2i + 1).
 
 x1 = x[:R/2], x2 = x[R/2:R]; o1 = x1*cos - x2*sin, o2 = x2*cos + x1*sin in 32-bit;
 dimensions from R on pass through: rollout/attention.py:10-25, rollout/fused.py:59-83.
@@ -22,6 +22,11 @@ class RotaryPosition:
         self.head_dim = int(params["head_dim"])
         self.rotary_dim = int(params.get("rotary_dim", self.head_dim))
         self.theta = float(params["theta"])
+        # which elements form a pair: "half" (i with i + R/2) or "interleaved" (2i with 2i + 1); the same
+        # angle table serves both, pair i turns by position * theta^(-2i/R)
+        self.pairing = params.get("pairing", "half")
+        if self.pairing not in ("half", "interleaved"):
+            raise ValueError(f"rotary pairing {self.pairing!r}: 'half' or 'interleaved'")
         # no limit of the model's own: as many positions as the engine's cache can hold for one request
         limit = params.get("max_position")
         self.max_position = int(limit if limit is not None else getattr(rt, "position_limit", 0) or 0)
@@ -48,6 +53,8 @@ class RotaryPosition:
 
     def apply(self, q, k, positions):
         """Rotate q and k ([T, heads, D], compute dtype) in place by their tokens' positions."""
+        if self.pairing != "half":
+            raise NotImplementedError("interleaved pairs are rotated by the mixers that prepare q and k with the tables")
         self.rt.ops.rope(q, positions, self.cos, self.sin, self.rotary_dim)
         if k is not None:
             self.rt.ops.rope(k, positions, self.cos, self.sin, self.rotary_dim)

@@ -51,6 +51,8 @@ Interfaces (``rt`` is the return_amd.parts.runtime.Runtime of the engine):
                 forward(x, step, tail) -> x + conv(x)   tail: [slots, rows, channels], updated in place
   token_input   something a layer adds to the stream for the token itself, after its other parts:
                 forward(h, pending, step)   h += pending (if any), then h += f(h, step.token_ids), in place
+  pass_input    what a looped stack does to the stream when a pass begins:
+                forward(h, pending, h0, number of the pass) -> (h, pending)   h0: the embedding's output
   embedding     forward(token_ids, step) -> h  fp32 [T, H]   (step.positions for absolute positions)
   head          forward(x) -> logits fp32 [rows, V]
 """
@@ -58,7 +60,8 @@ from __future__ import annotations
 
 from typing import Dict
 
-CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "input_conv", "token_input")
+CATEGORIES = ("norm", "mixer", "feed_forward", "position", "embedding", "head", "input_conv", "token_input",
+              "pass_input")
 _PARTS: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
 
 

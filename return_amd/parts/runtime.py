@@ -45,6 +45,26 @@ class Slabs:
         return self.tensor.shape[1:]
 
 
+class Scaled:
+    """A part's output that enters the residual stream times a factor: h += factor * tensor. A norm (or
+    whatever adds the pending output into the stream) takes it in place of the plain rows."""
+    __slots__ = ("tensor", "factor")
+
+    def __init__(self, tensor, factor):
+        self.tensor, self.factor = tensor, float(factor)
+
+    @property
+    def shape(self):
+        return self.tensor.shape
+
+
+def unscaled(delta):
+    """(rows, factor) of a pending output, Scaled or plain (None stays None)."""
+    if isinstance(delta, Scaled):
+        return delta.tensor, delta.factor
+    return delta, 1.0
+
+
 class ResidualSink:
     """Given to a part for its last product when what the product makes goes nowhere but into the
     residual stream, through a norm that takes every form of it: ``project(x, w)`` is x @ w^T in

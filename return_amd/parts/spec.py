@@ -59,11 +59,15 @@ class LayerCall:
     add_input: the embedding's output (the stream as it was before the first call) is added to
             the stream right before this call, as a looped stack does at the start of every pass
             but its first.
+    pass_input: number of the pass that begins with this call (0, 1, ...), for a model with a
+            ModelSpec.pass_input part: right before the call the stream becomes that part's function of
+            the stream, the embedding's output and the pass number. None: nothing is done.
     """
     block: int
     cache: Optional[object] = None
     writes_cache: bool = True
     add_input: bool = False
+    pass_input: Optional[int] = None
 
 
 @dataclasses.dataclass
@@ -79,6 +83,7 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     ignorable: List[str] = dataclasses.field(default_factory=list)  # tensors a checkpoint may hold unused
+    pass_input: Optional[PartSpec] = None   # what a looped stack does to the stream at the start of a pass (LayerCall.pass_input)
 
     def all_parts(self):
         """(category, where it sits, PartSpec) of every part of the model."""
@@ -90,6 +95,8 @@ class ModelSpec:
                 yield category, f"blocks[{i}].{name}", p
         yield "norm", "final_norm", self.final_norm
         yield "head", "head", self.head
+        if self.pass_input is not None:
+            yield "pass_input", "pass_input", self.pass_input
 
     def expected_tensors(self):
         """tensor name -> (shape, how the random-weights mode draws it)."""
