@@ -122,8 +122,9 @@ def expert(h, w, pre):
 
 def routed_feed_forward(h, w, pre, mlp):
     r = mlp["router"]
+    groups = r.get("groups") or {"count": 1, "keep": 1}                      # (no groups: one group of all)
     chosen, weights = route(h @ w[pre + "router"].T, w[pre + "correction"], int(r["top"]),
-                            int(r["groups"]["count"]), int(r["groups"]["keep"]))
+                            int(groups["count"]), int(groups["keep"]))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for e, a in zip(chosen[t].tolist(), weights[t]):

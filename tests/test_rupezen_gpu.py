@@ -1,0 +1,329 @@
+"""Rupezen on the GPU: every new kernel alone against its torch stand-in and against the plain
+implementation; inputs made so that one key decides (far back in the chunk, at page borders, just inside
+and just outside a chunk, in prompts and decoded alone); the engine against the plain model whole, with a
+decoded tail, in portions down to two tokens and in mixed batches with pages and slots used again, in both
+precisions; long decoding over several chunks; batches of unequal requests against each alone; greedy
+generation through Engine.generate with and without graphs; the trace program."""
+import os
+import types
+
+import pytest
+import torch
+
+from tests import trace_tools as tt
+from tests.plain import rupezen_plain as plain
+from tests.rupezen_cases import CASES, make_folder
+from tests.test_rupezen_cpu import _attention_weights, run_attention_in_pieces
+from tests.torch_ops import TorchOps
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from return_amd.kernels.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchOps(DEV)
+
+
+def tol(dtype):
+    return dict(atol=3e-5, rtol=3e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(v):
+    return torch.tensor(v, dtype=torch.int32, device=DEV)
+
+
+# ------------------------------------------------------------------ kernels alone
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,scale", [(1, 72, 0.7), (7, 256, 0.5), (40, 1000, 1.3), (3, 4096, 0.25), (300, 250, 0.9)])
+def test_norm_adds_a_scaled_delta_and_pass_rows(ops, ref, dtype, T, H, scale):
+    h_a, delta, w = rnd(T, H, seed=1), rnd(T, H, dtype=dtype, seed=2), rnd(H, seed=3).abs()
+    h_b = h_a.clone()
+    a, b = torch.empty(T, H, dtype=dtype, device=DEV), torch.empty(T, H, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h_a, delta, w, 1e-5, a, delta_scale=scale)
+    ref.add_rmsnorm(h_b, delta, w, 1e-5, b, delta_scale=scale)
+    torch.testing.assert_close(h_a, h_b, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    rows = i32(sorted({0, T // 2, T - 1}))
+    a, b = (torch.empty(rows.shape[0], H, dtype=dtype, device=DEV) for _ in range(2))
+    keep = h_a.clone()
+    ops.add_rmsnorm(h_a, delta, w, 1e-5, a, rows, delta_scale=scale)
+    ref.add_rmsnorm(h_b, delta, w, 1e-5, b, rows, delta_scale=scale)
+    torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    torch.testing.assert_close(h_a, keep, atol=0, rtol=0)              # with a row list the stream is left alone
+    h0 = rnd(T, H, seed=4)
+    for d in (delta, None):
+        a, b = (torch.empty(T, 2 * H, dtype=dtype, device=DEV) for _ in range(2))
+        ops.stream_pair_rows(h_a, d, scale, h0, a)
+        ref.stream_pair_rows(h_b, d, scale, h0, b)
+        torch.testing.assert_close(h_a, h_b, atol=1e-6, rtol=1e-6)
+        torch.testing.assert_close(a.float(), b.float(), atol=0 if dtype == torch.float32 else 2e-2, rtol=1e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,Dv,R,inter", [(4, 2, 8, 24, 4, True), (2, 1, 16, 8, 16, True), (6, 3, 4, 12, 0, True),
+                                                (3, 3, 10, 20, 10, False), (2, 2, 64, 128, 32, True), (1, 1, 5, 3, 2, True)])
+def test_maps_prepare(ops, ref, dtype, Hq, Hkv, D, Dv, R, inter):
+    T, P, pages = 37, 16, 5
+    qkv = rnd(T, (Hq + Hkv) * 2 * D + Hkv * Dv, dtype=dtype, seed=1)
+    pos = torch.randint(0, 200, (T,), generator=torch.Generator().manual_seed(2)).int().to(DEV)
+    ang = torch.outer(torch.arange(200).double(), 100.0 ** (-torch.arange(max(R // 2, 1)).double() * 2 / max(R, 1)))
+    cos, sin = (ang.cos().float().to(DEV), ang.sin().float().to(DEV)) if R else (None, None)
+    slots = torch.randperm(pages * P, generator=torch.Generator().manual_seed(3))[:T].int().to(DEV)
+    res = []
+    for o in (ops, ref):
+        q = torch.empty(T, Hq, 2 * D, dtype=dtype, device=DEV)
+        kp = torch.zeros(pages, Hkv, P, 2 * D, dtype=dtype, device=DEV)
+        vp = torch.zeros(pages, Hkv, P, Dv, dtype=dtype, device=DEV)
+        o.maps_qkv_prepare(qkv, Hq, Hkv, 2, D, Dv, pos, cos, sin, R, inter, q, kp, vp, slots)
+        res.append((q, kp, vp))
+    for a, b in zip(*res):
+        torch.testing.assert_close(a.float(), b.float(), **tol(dtype))
+    torch.testing.assert_close(res[0][2], res[1][2], atol=0, rtol=0)   # values are copied as they are
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("sizes", [(4, 2, 8, 24, 20, 4), (3, 3, 6, 7, None, 6), (2, 1, 10, 32, 16, 0), (2, 2, 16, 32, 33, 8),
+                                   (4, 1, 32, 48, 64, 32), (2, 1, 64, 128, 100, 16), (1, 1, 128, 64, 7, 64), (2, 2, 48, 96, 64, 12)])
+@pytest.mark.parametrize("pieces", [(150,), (118, *([1] * 32)), (7, 2, 24, 3, 64, 2, 5, 33, 9, 1)])
+def test_attention_in_pieces_equals_the_plain_function(ops, dtype, sizes, pieces):
+    H, G, D, V, chunk, R = sizes
+    g = torch.Generator().manual_seed(H * 100 + D)
+    T, W = sum(pieces), 24
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": 2.0 / D, "diff": 0.35}
+    if chunk:
+        m["mask"] = {"size": chunk}
+    if R:
+        m["rot"] = {"base": 100.0, "dims": R}
+    w = _attention_weights(g, W, H, G, D, V)
+    h = torch.randn(T, W, generator=g).double()
+    if dtype == torch.bfloat16:                         # the same rounded inputs on both sides
+        h = h.bfloat16().double()
+        w = {k: v.bfloat16().double() for k, v in w.items()}
+    want = plain.differential_attention(h, w, "", m, 1e-5)
+    got = run_attention_in_pieces(ops, h, w, m, 1e-5, pieces, pages=tuple(torch.randperm(12, generator=g).tolist()),
+                                  dtype=dtype, device=DEV)
+    if dtype == torch.float32:
+        torch.testing.assert_close(got.double().cpu(), want, atol=2e-4, rtol=2e-4)
+    else:
+        # the normed output has a root mean square of 1 - diff: rows are held by their error against that
+        err = (got.double().cpu() - want).pow(2).mean(-1).sqrt()
+        assert float(err.max()) < 0.04, f"row {int(err.argmax())}: {float(err.max()):.3e}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("D,V,C", [(8, 8, 10), (16, 32, 32), (64, 128, 48), (48, 96, 64)])
+@pytest.mark.parametrize("pieces_of", ["prompt", "decoded"])
+def test_one_key_decides_at_the_chunk_borders(ops, dtype, D, V, C, pieces_of):
+    """Two keys with large values sit on the first and on the last place of a chunk (a page's first and last
+    row where the sizes allow). Queries made to look their way read them from inside the chunk, right behind
+    them and from the chunk's far end, and not from the next chunk, first place or later."""
+    g = torch.Generator().manual_seed(D)
+    W, H, G = 16, 2, 1
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": 8.0 / D, "diff": 0.5, "mask": {"size": C}}
+    w = _attention_weights(g, W, H, G, D, V)
+    T = 3 * C + 5
+    h = 0.05 * torch.randn(T, W, generator=g).double()
+    spot = 2 * C - 1                                   # the last key of the second chunk
+    h[C] *= 80.0                                       # and its first
+    h[spot] = h[C] * 0.9
+    for at in (C + 1, spot - 1, spot + 1, spot + 2, 3 * C - 1, 3 * C):
+        h[at] = h[C] * 0.3                             # (their own keys are small beside the two)
+    if dtype == torch.bfloat16:
+        h = h.bfloat16().double()
+        w = {k: v.bfloat16().double() for k, v in w.items()}
+    want = plain.differential_attention(h, w, "", m, 1e-6)
+    open_mask = dict(m)
+    open_mask.pop("mask")
+    assert (plain.differential_attention(h, w, "", open_mask, 1e-6)[spot + 1] - want[spot + 1]).abs().max() > 0.05
+    pieces = (T,) if pieces_of == "prompt" else (C - 3, *([1] * (T - C + 3)))
+    got = run_attention_in_pieces(ops, h, w, m, 1e-6, pieces, pages=tuple(torch.randperm(3 * C // 16 + 2, generator=g).tolist()),
+                                  dtype=dtype, device=DEV).double().cpu()
+    err = (got - want).pow(2).mean(-1).sqrt()
+    limit = 2e-4 if dtype == torch.float32 else 0.04
+    assert float(err.max()) < limit, f"query at {int(err.argmax())} (chunk of {C}, key at {spot}): {float(err.max()):.3e}"
+
+
+@pytest.mark.parametrize("T,E,top,count,keep", [(1, 8, 2, 4, 2), (40, 6, 3, 2, 1), (33, 5, 1, 1, 1), (17, 6, 2, 6, 3),
+                                                (300, 9, 4, 3, 2), (64, 256, 8, 8, 4), (5, 70, 6, 1, 1), (9, 4, 4, 1, 1)])
+def test_router_kernel_equals_the_plain_choice(ops, T, E, top, count, keep):
+    g = torch.Generator().manual_seed(E * 10 + top)
+    z = 2.0 * torch.randn(T, E, generator=g)
+    corr = 0.5 * torch.randn(E, generator=g)
+    want_ids, want_w = plain.route(z.double(), corr.double(), top, count, keep)
+    ids, w = ops.moe_route(z.to(DEV), corr.to(DEV), top, count, keep, 1e-20)
+    assert ids.cpu().long().tolist() == want_ids.tolist()
+    torch.testing.assert_close(w.cpu().double(), want_w, atol=1e-6, rtol=1e-5)
+    ids, _ = ops.moe_route(z.to(DEV), None, top, count, keep, 1e-20)
+    assert ids.cpu().long().tolist() == plain.route(z.double(), torch.zeros(E).double(), top, count, keep)[0].tolist()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,H,I,E,top", [(1, 64, 24, 8, 2), (9, 72, 20, 6, 3), (37, 64, 40, 5, 1), (300, 96, 64, 4, 2),
+                                        (700, 128, 32, 8, 2), (3, 50, 13, 7, 7), (64, 256, 100, 64, 6)])
+def test_experts_kernels_equal_the_stand_in(ops, ref, dtype, T, H, I, E, top):
+    x = rnd(T, H, dtype=dtype, seed=1)
+    gate_up = rnd(E, 2 * I, H, dtype=dtype, seed=2, scale=H ** -0.5)
+    down = rnd(E, H, I, dtype=dtype, seed=3, scale=I ** -0.5)
+    g = torch.Generator().manual_seed(4)
+    ids = torch.stack([torch.randperm(E, generator=g)[:top] for _ in range(T)]).int().to(DEV)
+    if T >= 300:
+        ids[: T // 2, 0] = 1                            # many rows for one expert: full tiles and a ragged last one
+    weights = torch.rand(T, top, generator=g).to(DEV)
+    got = ops.moe_experts(x, ids, weights, gate_up, down)
+    want = ref.moe_experts(x, ids, weights, gate_up, down)
+    torch.testing.assert_close(got.float(), want.float(), **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32
+                                                            else dict(atol=3e-2, rtol=3e-2)))
+
+
+# ------------------------------------------------------------------ the engine against the plain model
+LENGTHS = {"a": 5, "b": 17, "c": 33, "d": 100, "e": 64, "f": 150, "g": 1, "h": 47}
+# A row's error: the root mean square over the vocabulary of the difference of the logits, its mean taken off,
+# over the root mean square of the plain logits. bfloat16 rows are also held against a stand-in engine of torch
+# operations that rounds where the kernels round.
+ROW_ERROR = {"float32": 5e-5, "bfloat16": 0.3}
+ROW_ERROR_16_MEAN = 0.04
+ROW_ERROR_16_STAND_IN = 0.1
+
+
+@pytest.fixture(scope="module", params=sorted(CASES))
+def model(request, tmp_path_factory):
+    folder = make_folder(tmp_path_factory, request.param)
+    cfg, w = plain.read_folder(folder)
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in LENGTHS.items()}
+    want = {rid: plain.logits(cfg, w, toks) for rid, toks in reqs.items()}
+    steps = tt.whole(reqs)
+    rounded = tt.run_in_process(make_runner(folder, "bfloat16", tt.peak_tokens(steps), ops=TorchOps(DEV)), steps)
+    return folder, cfg, reqs, want, rounded
+
+
+def make_runner(folder, dtype, max_tokens, page=16, ops=None, **kw):
+    from return_amd.config import EngineConfig
+    from return_amd.engine import ModelRunner
+    ec = EngineConfig(dtype=dtype, page_size=page, max_token=max_tokens, max_reside=4, max_step_tokens=max(max_tokens, 4),
+                      prefill_chunk=max_tokens, tune_products=False, check_invariants=True, **kw)
+    return ModelRunner(folder, engine_config=ec, ops=ops)
+
+
+def row_error(a, b):
+    d = (a - b).double()
+    return float((d - d.mean()).pow(2).mean().sqrt() / b.double().pow(2).mean().sqrt())
+
+
+def compare(got, want, reqs, dtype, rounded=None):
+    worst, total, n = 0.0, 0.0, 0
+    for rid, toks in reqs.items():
+        for p in range(len(toks)):
+            e = row_error(got[(rid, p)], want[rid][p])
+            worst, total, n = max(worst, e), total + e, n + 1
+            assert e <= ROW_ERROR[dtype], f"request {rid} position {p} (first wrong place): row error {e:.3e}"
+            if dtype == "bfloat16" and rounded is not None:
+                e16 = row_error(got[(rid, p)], rounded[(rid, p)])
+                assert e16 <= ROW_ERROR_16_STAND_IN, \
+                    f"request {rid} position {p} (first wrong place): {e16:.3e} from the stand-in that rounds alike"
+    if dtype == "bfloat16":
+        assert total / n <= ROW_ERROR_16_MEAN, f"mean row error {total / n:.3e}"
+    return worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("cut", ["whole", "tail_decoded", "portions", "mixed"])
+def test_engine_matches_plain(model, dtype, cut):
+    folder, cfg, reqs, want, rounded = model
+    steps = {"whole": tt.whole, "tail_decoded": tt.tail_decoded, "portions": tt.portions, "mixed": tt.mixed}[cut](reqs)
+    runner = make_runner(folder, dtype, tt.peak_tokens(steps))
+    got = tt.run_in_process(runner, steps)
+    print(f"rupezen {dtype} {cut}: largest row error {compare(got, want, reqs, dtype, rounded):.2e}")
+    assert not runner.cache.live and all(g.pages.in_use() == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page", [4, 64])
+def test_long_decoding_passes_many_chunks(tmp_path_factory, dtype, page):
+    """A short prompt and 280 tokens one by one: every chunk border is crossed by decoded tokens, and pages
+    of chunks that are over go back to the pool while the request runs (pages smaller and larger than the chunks)."""
+    folder = make_folder(tmp_path_factory, "a")
+    cfg, w = plain.read_folder(folder)
+    toks = tt.random_tokens(cfg["vocab"], 300, seed=4)
+    steps = tt.tail_decoded({"r": toks}, tail=280)
+    runner = make_runner(folder, dtype, 320, page=page)
+    got = tt.run_in_process(runner, steps)
+    print(f"rupezen {dtype} long decoding: largest row error "
+          f"{compare(got, {'r': plain.logits(cfg, w, toks)}, {'r': toks}, dtype):.2e}")
+
+
+def test_batches_of_unequal_requests_equal_each_alone(tmp_path_factory):
+    folder = make_folder(tmp_path_factory, "b")
+    cfg, _ = plain.read_folder(folder)
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in (("a", 70), ("b", 3), ("c", 41), ("d", 1))}
+    sizes = {"a": [30, 1, 1, 38], "b": [1, 2], "c": [2, 39], "d": [1]}
+    for dtype, limit in (("float32", 2e-5), ("bfloat16", 0.05)):
+        alone = {}
+        for rid, toks in reqs.items():
+            alone.update(tt.run_in_process(make_runner(folder, dtype, 256), tt.portions({rid: toks}, sizes=tuple(sizes[rid]))))
+        steps, at = [], {rid: 0 for rid in reqs}
+        for k in range(4):
+            entries, end = [], []
+            for rid, toks in reqs.items():
+                if k < len(sizes[rid]):
+                    n = sizes[rid][k]
+                    entries.append({"id": rid, "tokens": toks[at[rid]:at[rid] + n], "want": list(range(n))})
+                    at[rid] += n
+                    if at[rid] == len(toks):
+                        end.append(rid)
+            steps.append({"step": k, "entries": entries, "end": end})
+        together = tt.run_in_process(make_runner(folder, dtype, 256), steps)
+        for key, row in alone.items():
+            assert row_error(together[key], row) < limit, (dtype, key)
+
+
+# ------------------------------------------------------------------ generation and the programs
+def test_greedy_generation_through_the_engine(tmp_path_factory):
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    for name in ("a", "c"):
+        folder = make_folder(tmp_path_factory, name)
+        cfg, w = plain.read_folder(folder)
+        prompts = [tt.random_tokens(cfg["vocab"], n, seed=n) for n in (1, 8, 31, 64, 90)]
+        want = [plain.greedy_generate(cfg, w, p, 12) for p in prompts]
+        for graphs in (False, True):
+            eng = Engine(folder, dtype="float32", page_size=16, max_token=1024, max_reside=4, max_step_tokens=64,
+                         prefill_chunk=24, use_graphs=graphs, check_invariants=True)
+            got = eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=12))
+            assert [r.output_ids for r in got] == want, f"model {name}, graphs {graphs}"
+            assert not eng.runner.cache.live
+
+
+def test_bf16_generation_from_graphs_equals_eager(tmp_path_factory):
+    from return_amd import SamplingParams
+    from return_amd.engine import Engine
+    folder = make_folder(tmp_path_factory, "c")
+    cfg, _ = plain.read_folder(folder)
+    prompts = [tt.random_tokens(cfg["vocab"], n, seed=n) for n in (3, 40, 77)]
+    outs = []
+    for graphs in (False, True):
+        eng = Engine(folder, dtype="bfloat16", page_size=16, max_token=1024, max_reside=4, use_graphs=graphs)
+        outs.append([r.output_ids for r in eng.generate(prompts, SamplingParams(temperature=0.0, max_new_tokens=24))])
+    assert outs[0] == outs[1]
+
+
+def test_trace_program_on_a_model_folder(tmp_path_factory, tmp_path):
+    folder = make_folder(tmp_path_factory, "b")
+    cfg, w = plain.read_folder(folder)
+    reqs = {rid: tt.random_tokens(cfg["vocab"], n, seed=ord(rid)) for rid, n in (("a", 40), ("b", 7), ("c", 90))}
+    steps = tt.mixed(reqs, seed=3, max_live=3)
+    got = tt.run_program(folder, "float32", steps, str(tmp_path), tt.peak_tokens(steps), cfg["vocab"],
+                         env=dict(os.environ))
+    compare(got, {rid: plain.logits(cfg, w, t) for rid, t in reqs.items()}, reqs, "float32")

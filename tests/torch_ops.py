@@ -13,6 +13,11 @@ import torch
 from return_amd.parts.runtime import ScaledRows, Slabs
 
 
+def _pool_rows(pool, pages, n):
+    """The first n token rows that the listed pages of a pool [pages, kv heads, rows in a page, width] hold, [n, kv heads, width]."""
+    return pool[pages].transpose(1, 2).reshape(-1, pool.shape[1], pool.shape[3])[:n].float()
+
+
 class TorchOps:
     def __init__(self, device="cpu"):
         self.device = torch.device(device)
@@ -22,22 +27,27 @@ class TorchOps:
         out.copy_(table[ids.long()].float())
 
     # rollout/fused.py:6-17 with the residual addition of qwen3.py:63,67 in front
-    def add_rmsnorm(self, h, delta, weight, eps, out, rows=None):
+    def add_rmsnorm(self, h, delta, weight, eps, out, rows=None, delta_scale=1.0):
         if isinstance(delta, Slabs):                        # shares of a product: their sum, rounded as the product would be
             delta = delta.tensor.sum(0).to(out.dtype)
         if rows is None:
             if delta is not None:
-                h += delta.float()
+                h += delta_scale * delta.float()
             v = h
         else:
             v = h[rows.long()]
             if delta is not None:
-                v = v + delta[rows.long()].float()
+                v = v + delta_scale * delta[rows.long()].float()
         rstd = 1.0 / torch.sqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
         out.copy_((v * rstd * weight).to(out.dtype))
 
-    def residual_add(self, h, delta):
-        h += delta.float()
+    def residual_add(self, h, delta, scale=1.0):
+        h += scale * delta.float()
+
+    def stream_pair_rows(self, h, delta, delta_scale, h0, out):
+        if delta is not None:
+            h += delta_scale * delta.float()
+        out.copy_(torch.cat([h, h0], dim=1).to(out.dtype))
 
     # rollout/fused.py:36-56 on a [-1, D] view
     def head_rmsnorm(self, x, weight, eps):
@@ -177,6 +187,89 @@ class TorchOps:
             else:
                 prob = score.softmax(-1)
             out[a:b] = torch.einsum("hqk,khd->qhd", prob, vv).to(out.dtype)
+
+    # ---- attention with two score maps per head over the same values
+    def maps_qkv_prepare(self, qkv, n_q, n_kv, maps, D, Dv, positions, cos, sin, rotary_dim, interleaved, q_out,
+                         k_pool, v_pool, slot_mapping):
+        T, R = qkv.shape[0], int(rotary_dim)
+        qw, kw = n_q * maps * D, n_kv * maps * D
+        q = qkv[:, :qw].reshape(T, n_q * maps, D).float()
+        k = qkv[:, qw:qw + kw].reshape(T, n_kv * maps, D).float()
+        v = qkv[:, qw + kw:].reshape(T, n_kv, Dv)
+
+        def rot(x):
+            if R == 0:
+                return x
+            c, s = cos[positions.long()][:, None, :], sin[positions.long()][:, None, :]
+            if interleaved:
+                u, w = x[..., 0:R:2], x[..., 1:R:2]
+                turned = torch.stack([u * c - w * s, w * c + u * s], dim=-1).reshape(*x.shape[:-1], R)
+            else:
+                u, w = x[..., :R // 2], x[..., R // 2:R]
+                turned = torch.cat([u * c - w * s, w * c + u * s], dim=-1)
+            return torch.cat([turned, x[..., R:]], dim=-1)
+
+        q_out.copy_(rot(q).reshape(T, n_q, maps * D).to(q_out.dtype))
+        if k_pool is not None:
+            P = k_pool.shape[2]
+            page, row = slot_mapping.long() // P, slot_mapping.long() % P
+            k_pool[page, :, row] = rot(k).reshape(T, n_kv, maps * D).to(k_pool.dtype)
+            v_pool[page, :, row] = v
+
+    def attention_diff(self, q, out, k_pool, v_pool, step, group, scale, lam, eps, out_scale, window=0, chunk=0):
+        g = step.groups[group]
+        n_q, n_kv, D = q.shape[1], k_pool.shape[1], q.shape[2] // 2
+        cu_q, cu_p = step.cu_q.tolist(), g.cu_pages.tolist()
+        q_start, kv_start = step.q_start.tolist(), g.kv_start.tolist()
+        table = g.page_table.long()
+        for s in range(step.n_seqs):
+            a, b = cu_q[s], cu_q[s + 1]
+            pages = table[cu_p[s]:cu_p[s + 1]]
+            end = q_start[s] + (b - a)
+            k = _pool_rows(k_pool, pages, end - kv_start[s]).repeat_interleave(n_q // n_kv, dim=1)
+            v = _pool_rows(v_pool, pages, end - kv_start[s]).repeat_interleave(n_q // n_kv, dim=1)
+            k_pos = torch.arange(kv_start[s], end, device=q.device)
+            q_pos = torch.arange(q_start[s], end, device=q.device)
+            hide = k_pos[None, :] > q_pos[:, None]
+            if window:
+                hide = hide | (k_pos[None, :] <= q_pos[:, None] - window)
+            if chunk:
+                hide = hide | (k_pos[None, :] // chunk != q_pos[:, None] // chunk)
+            qq = q[a:b].float()
+            maps = []
+            for m in range(2):
+                score = torch.einsum("qhd,khd->hqk", qq[..., m * D:(m + 1) * D], k[..., m * D:(m + 1) * D]) * scale
+                maps.append(torch.einsum("hqk,khd->qhd", score.masked_fill(hide[None], float("-inf")).softmax(-1), v))
+            o = maps[0] - lam * maps[1]
+            o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * out_scale
+            out[a:b] = o.to(out.dtype)
+
+    # ---- routed experts
+    def moe_route(self, z, bias, top, groups, keep, norm_eps):
+        T, E = z.shape
+        s = torch.sigmoid(z.float())
+        c = s + (bias if bias is not None else 0.0)
+        if groups > 1 and keep < groups:
+            per = E // groups
+            score = c.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+            stay = torch.zeros(T, groups, dtype=torch.bool, device=z.device)
+            stay.scatter_(1, score.topk(keep, dim=-1).indices, True)
+            c = c.masked_fill(~stay[:, :, None].expand(T, groups, per).reshape(T, E), float("-inf"))
+        ids = c.topk(top, dim=-1).indices
+        w = s.gather(1, ids)
+        return ids.int(), w / (w.sum(-1, keepdim=True) + norm_eps)
+
+    def moe_experts(self, x, ids, weights, w_gate_up, w_down):
+        T, H = x.shape
+        I = w_gate_up.shape[1] // 2
+        out = torch.zeros(T, H, dtype=torch.float32, device=x.device)
+        for t in range(T):
+            for k in range(ids.shape[1]):
+                e = int(ids[t, k])
+                gu = (x[t].float() @ w_gate_up[e].float().t()).to(x.dtype).float()
+                a = (gu[:I] * torch.sigmoid(gu[:I]) * gu[I:]).to(x.dtype)
+                out[t] += weights[t, k] * (a.float() @ w_down[e].float().t()).to(x.dtype).float()
+        return out.to(x.dtype)
 
     # ---- the parts beside the usual ones, each as its kernel is called
     def relu_sq(self, x):
