@@ -94,8 +94,8 @@ __global__ __launch_bounds__(WAVES * 64) void attn_diff_plain_kernel(
     const T* __restrict__ v_pool, const int* __restrict__ page_table,
     const int* __restrict__ cu_pages, const int* __restrict__ kv_start,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
-    const int* __restrict__ tok_ids, int n_seqs, int T_tokens, int Hq, int Hkv, int D, int Dv, int P,
-    float scale, int window, int chunk, float lambda, float eps, float out_scale) {
+    const int* __restrict__ tok_ids, int ids_are_requests, int n_seqs, int T_tokens, int Hq, int Hkv, int D, int Dv,
+    int P, float scale, int window, int chunk, float lambda, float eps, float out_scale) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
     const int D2 = 2 * D;
     float* q_s = smem;                                   // [QR][2D]
@@ -116,11 +116,18 @@ __global__ __launch_bounds__(WAVES * 64) void attn_diff_plain_kernel(
         const int qi = blockIdx.x * QR + r;
         t_of[r] = seg_of[r] = pos_of[r] = 0;
         if (qi < T_tokens) {
-            const int t = tok_ids ? tok_ids[qi] : qi;
-            int lo = 0, hi = n_seqs - 1;
-            while (lo < hi) {
-                const int mid = (lo + hi + 1) >> 1;
-                if (cu_q[mid] <= t) lo = mid; else hi = mid - 1;
+            int t, lo;
+            if (tok_ids != nullptr && ids_are_requests) {          // the list names requests that bring one token each
+                lo = tok_ids[qi];
+                t = cu_q[lo];
+            } else {
+                t = tok_ids ? tok_ids[qi] : qi;
+                lo = 0;
+                int hi = n_seqs - 1;
+                while (lo < hi) {
+                    const int mid = (lo + hi + 1) >> 1;
+                    if (cu_q[mid] <= t) lo = mid; else hi = mid - 1;
+                }
             }
             todo |= 1u << r;
             t_of[r] = t;
@@ -324,14 +331,14 @@ static size_t diff_plain_floats(int QR, int WAVES, int D, int Dv) {
 template <typename T, int QR, int WAVES>
 static void diff_plain_launch(hipStream_t st, const void* q, void* out, const void* k_pool, const void* v_pool,
                               const int* page_table, const int* cu_pages, const int* kv_start, const int* cu_q,
-                              const int* q_start, const int* tok_ids, int n_seqs, int T_tokens, int Hq, int Hkv,
-                              int D, int Dv, int P, float scale, int window, int chunk, float lambda, float eps,
-                              float out_scale) {
+                              const int* q_start, const int* tok_ids, int ids_are_requests, int n_seqs, int T_tokens,
+                              int Hq, int Hkv, int D, int Dv, int P, float scale, int window, int chunk, float lambda,
+                              float eps, float out_scale) {
     dim3 grid((T_tokens + QR - 1) / QR, Hq), block(WAVES * 64);
     hipLaunchKernelGGL((attn_diff_plain_kernel<T, QR, WAVES>), grid, block, diff_plain_floats(QR, WAVES, D, Dv) * sizeof(float),
                        st, (const T*)q, (T*)out, (const T*)k_pool, (const T*)v_pool, page_table, cu_pages, kv_start,
-                       cu_q, q_start, tok_ids, n_seqs, T_tokens, Hq, Hkv, D, Dv, P, scale, window, chunk, lambda, eps,
-                       out_scale);
+                       cu_q, q_start, tok_ids, ids_are_requests, n_seqs, T_tokens, Hq, Hkv, D, Dv, P, scale, window, chunk,
+                       lambda, eps, out_scale);
 }
 
 // Whether the plain kernel takes these sizes (its LDS holds a row's query maps and the waves' sums).
@@ -341,18 +348,21 @@ extern "C" int ra_attention_diff_plain_fits(int D, int Dv) {
 
 extern "C" int ra_attention_diff_plain(const void* q, void* out, const void* k_pool, const void* v_pool,
                                        const int* page_table, const int* cu_pages, const int* kv_start,
-                                       const int* cu_q, const int* q_start, const int* tok_ids, int n_seqs,
-                                       int T_tokens, int Hq, int Hkv, int D, int Dv, int P, float scale, int window,
+                                       const int* cu_q, const int* q_start, const int* tok_ids,
+                                       int ids_are_requests, int n_seqs, int T_tokens, int Hq, int Hkv, int D, int Dv, int P, float scale, int window,
                                        int chunk, float lambda, float eps, float out_scale, int dtype, void* stream) {
     if (T_tokens <= 0 || n_seqs <= 0) return RA_OK;
     if (!ra_attention_diff_plain_fits(D, Dv) || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 || Hq > 65535) return RA_ERR_ARG;
     if (dtype != RA_DTYPE_F32 && dtype != RA_DTYPE_BF16) return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    const bool single = tok_ids == nullptr && T_tokens == n_seqs;
+    // tok_ids: the rows of q to work on (null: all T_tokens rows), or, with ids_are_requests, the numbers of
+    // requests that bring one token each (their rows are cu_q[request])
+    const bool single = (tok_ids == nullptr && T_tokens == n_seqs) || (tok_ids != nullptr && ids_are_requests);
     const size_t limit = 65536 / sizeof(float);
 #define DIFF_GO(T_, QR_, W_)                                                                                  \
     diff_plain_launch<T_, QR_, W_>(st, q, out, k_pool, v_pool, page_table, cu_pages, kv_start, cu_q, q_start,  \
-                                   tok_ids, n_seqs, T_tokens, Hq, Hkv, D, Dv, P, scale, window, chunk, lambda, eps, out_scale)
+                                   tok_ids, ids_are_requests, n_seqs, T_tokens, Hq, Hkv, D, Dv, P, scale, window, chunk,  \
+                                   lambda, eps, out_scale)
 #define DIFF_PICK(T_)                                                                                         \
     do {                                                                                                      \
         if (single && diff_plain_floats(1, 8, D, Dv) <= limit) DIFF_GO(T_, 1, 8);                             \

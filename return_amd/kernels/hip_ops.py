@@ -55,7 +55,9 @@ def _declare(lib):
         "ra_add_scaled_rmsnorm": [P, P, F, P, F, P, P, I, I, I, P],
         "ra_stream_pair_rows": [P, P, F, P, P, L, I, I, P],
         "ra_maps_qkv_prepare": [P, I, I, I, I, I, I, P, P, P, I, I, P, P, P, P, I, I, P],
-        "ra_attention_diff_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, F, F, F, I, P],
+        "ra_attention_diff_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, F, F, I, P],
+        "ra_attention_diff_mfma_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, F, F, F, P],
+        "ra_attention_diff_mfma_fits": [I, I],
         "ra_attention_diff_plain_fits": [I, I],
         "ra_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
         "ra_moe_plan": [P, I, I, I, P, P, P, P],
@@ -1230,6 +1232,8 @@ class HipOps:
     def diff_prefill_tile_rows(self, D, Dv, dtype):
         """Rows per q tile of the lists that attention_diff reads from step.prefill_tiles, or None where the
         kernel that serves these sizes takes no list."""
+        if dtype == torch.bfloat16 and self.lib.ra_attention_diff_mfma_fits(int(D), int(Dv)):
+            return (64,)
         return None
 
     def attention_diff(self, q, out, k_pool, v_pool, step, group, scale, lam, eps, out_scale, window=0, chunk=0):
@@ -1247,10 +1251,26 @@ class HipOps:
         self.check_attention_diff_sizes(n_q, n_kv, D2 // 2, Dv, q.dtype)
         P = k_pool.shape[2]
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
-        self._check(self.lib.ra_attention_diff_plain(
-            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, None, step.n_seqs, T, n_q, n_kv, D2 // 2, Dv, P,
-            float(scale), int(window), int(chunk), float(lam), float(eps), float(out_scale), _code(q.dtype),
-            self._stream()), "attention_diff_plain")
+        consts = (float(scale), int(window), int(chunk), float(lam), float(eps), float(out_scale))
+
+        def plain(ids, ids_are_requests, rows):
+            self._check(self.lib.ra_attention_diff_plain(
+                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(ids), 1 if ids_are_requests else 0,
+                step.n_seqs, rows, n_q, n_kv, D2 // 2, Dv, P, *consts, _code(q.dtype), self._stream()),
+                "attention_diff_plain")
+
+        tiles = step.prefill_tiles.get(64) if getattr(step, "prefill_tiles", None) else None
+        if tiles is not None and step.n_prefill_tokens > 0 and q.dtype == torch.bfloat16 and scale > 0 and \
+                self.lib.ra_attention_diff_mfma_fits(D2 // 2, Dv):
+            # requests with two or more new tokens on the matrix cores, tile by tile; the others (one token
+            # each) by the plain kernel, a workgroup of eight waves over the keys of each
+            self._check(self.lib.ra_attention_diff_mfma_bf16(
+                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], n_q, n_kv,
+                D2 // 2, Dv, P, *consts, self._stream()), "attention_diff_mfma_bf16")
+            if step.n_decode > 0:
+                plain(step.decode_segs, True, step.n_decode)
+            return
+        plain(None, False, T)
 
     # ------------------------------------------------------------------ routed experts
     MAX_EXPERTS = 1024

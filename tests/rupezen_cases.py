@@ -51,7 +51,7 @@ RUPE_C = {
     "loop": {"start": 0, "stop": 2, "times": 3},
     "layers": [
         _layer(4, 2, 16, 32, 0.25, 0.5, chunk=16, rot=(10000.0, 8), moe=(32, 8, 2, 2, 1)),
-        _layer(2, 1, 32, 48, 0.18, 0.35, chunk=40, rot=(10000.0, 32), moe=(64, 4, 2, 1, 1)),
+        _layer(2, 1, 32, 96, 0.18, 0.35, chunk=40, rot=(10000.0, 32), moe=(64, 4, 2, 1, 1)),
     ]}
 RUPE_C_INIT = dict(seed=23, std=0.12, embedding_std=1.0, norm_jitter=0.05)
 
