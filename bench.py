@@ -671,11 +671,147 @@ def kofipel(args):
             "measured": peaks, "designs": out}
 
 
+# The Rupezen design beside the Qwen3 design at equal sizes: --workload rupezen
+def rupezen_shape(width, heads, kv_heads, head_dim, ff, layers, vocab, experts=32, top=4, chunk=4096):
+    """config.json of a Rupezen model: `layers` layers of which the two in the middle run twice (layers + 2 runs),
+    two score maps of head_dim / 2 per head (a key row as wide as the Qwen3 head), values of head_dim, experts of
+    ff / top channels each (as many active channels as the dense feed-forward)."""
+    layer = {"type": "attention",
+             "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": head_dim // 2, "vdim": head_dim, "diff": 0.5,
+                       "scale": (head_dim // 2) ** -0.5, "mask": {"size": chunk},
+                       "rot": {"base": 1e6, "dims": head_dim // 4}},
+             "mlp": {"kind": "moe", "expert": {"ff": ff // top},
+                     "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}}
+    mid = layers // 2
+    return {"architecture": "Rupezen", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 0.5,
+            "loop": {"start": mid - 1, "stop": mid + 1, "times": 2}, "layers": [layer] * layers}
+
+
+def rupezen_runs(raw):
+    """Layer numbers in the order they run."""
+    n, loop = len(raw["layers"]), raw.get("loop")
+    if not loop:
+        return list(range(n)), 0
+    inner = list(range(loop["start"], loop["stop"]))
+    return list(range(loop["start"])) + inner * loop["times"] + list(range(loop["stop"], n)), loop["times"]
+
+
+def rupezen_bytes(raw, elt, batch, ctx):
+    """Bytes one decode step has to move: every matrix of a layer run once (of the experts those that the step's
+    tokens are expected to choose, every token choosing `top` of them evenly), the keys and values of the chunk
+    that the context ends in, the head."""
+    W = raw["width"]
+    runs, passes = rupezen_runs(raw)
+    total = raw["vocab"] * W * elt + passes * 2 * W * W * elt
+    for i in runs:
+        m, mlp = raw["layers"][i]["mixer"], raw["layers"][i]["mlp"]
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        total += ((H + G) * 2 * D + G * V + H * V) * W * elt
+        seen = ctx % m["mask"]["size"] + 1 if m.get("mask") else ctx
+        total += batch * seen * G * (2 * D + V) * elt
+        if mlp:
+            E, top = mlp["router"]["experts"], mlp["router"]["top"]
+            chosen = E * (1.0 - (1.0 - top / E) ** batch)
+            total += (E * W + chosen * 3 * W * mlp["expert"]["ff"]) * elt
+    return total
+
+
+def rupezen_flops(raw, T):
+    """Operations of a prompt of T tokens on the matrix cores: the products (of the experts the chosen ones), both
+    score maps and both sums over the values inside the chunks (the weights' second halves not counted)."""
+    W = raw["width"]
+    runs, passes = rupezen_runs(raw)
+    lin = raw["vocab"] * W / T + passes * 2 * W * W
+    attn = 0.0
+    for i in runs:
+        m, mlp = raw["layers"][i]["mixer"], raw["layers"][i]["mlp"]
+        H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+        lin += ((H + G) * 2 * D + G * V + H * V) * W
+        c = m["mask"]["size"] if m.get("mask") else T
+        keys = sum(t % c + 1 for t in range(T))
+        attn += keys * H * (4.0 * D + 4.0 * V)
+        if mlp:
+            lin += mlp["router"]["experts"] * W + mlp["router"]["top"] * 3 * W * mlp["expert"]["ff"]
+    return 2.0 * T * lin + attn
+
+
+def rupezen(args):
+    """Prefill of 2,048 tokens and decode at batch 1, 8 and 64 over 2,048-token prefixes of the Rupezen design at
+    two sizes that resemble a model's layers (eight layer runs, random weights), each beside the Qwen3 design with
+    the same width, heads, key row, active feed-forward width and number of layer runs, through the same engine;
+    the step's time by kernel for both. value: Rupezen decode tok/s at batch 8 on the larger size."""
+    import torch
+    from return_amd.engine.runner import StepEntry
+    elt = 2 if args.dtype == "bfloat16" else 4
+    runs, vocab = 8, 32000
+    sizes = {"w2048": dict(width=2048, heads=16, kv_heads=4, head_dim=128, ff=8192),
+             "w4096": dict(width=4096, heads=32, kv_heads=8, head_dim=128, ff=12288)}
+    k, w = max(8, min(args.steps, 32)), min(args.warmup, 4)
+    out, peaks = {}, None
+    for tag, sz in sizes.items():
+        raws = {"rupezen": rupezen_shape(layers=runs - 2, vocab=vocab, **sz),
+                "qwen3": dict(QWEN3_8B, vocab_size=vocab, hidden_size=sz["width"], num_hidden_layers=runs,
+                              num_attention_heads=sz["heads"], num_key_value_heads=sz["kv_heads"],
+                              head_dim=sz["head_dim"], intermediate_size=sz["ff"])}
+        for design, raw in raws.items():
+            cfg, runner = build_runner(0, args.dtype, 64, raw=raw, std=0.02, use_graphs=not args.no_graphs,
+                                       tune_products=not args.no_tune, defer_norms=not args.no_defer_norms)
+            if peaks is None:
+                peaks = measured_peaks(runner, args.dtype)
+            rec = {}
+            toks = [(7 * i + 3) % vocab for i in range(PREFILL_TOKENS)]
+
+            def prompt():
+                runner.add_request("p")
+                runner.step([StepEntry("p", toks, [PREFILL_TOKENS - 1])])
+                runner.free_request("p")
+            prompt()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(3):
+                prompt()
+            torch.cuda.synchronize()
+            secs = (time.perf_counter() - t0) / 3
+            rec["prefill_2048"] = prefill_record(cfg, args.dtype, PREFILL_TOKENS, secs, peaks=peaks,
+                                                 flops=rupezen_flops(raw, PREFILL_TOKENS) if design == "rupezen" else None)
+            rec["prefill_2048"]["kernels"] = kernel_split(prompt, 2)
+            for b in (1, 8, 64):
+                ids = seat_requests(runner, b, CONTEXT)
+                secs = decode_steps(runner, ids, k, w, vocab)
+                ms = secs / k * 1e3
+                point = {"tok_s": round(b * k / secs, 1), "ms_per_step": round(ms, 4)}
+                if design == "rupezen":
+                    got = rupezen_bytes(raw, elt, b, CONTEXT + w + (k + 1) // 2) / (ms * 1e-3) / 1e9
+                    point.update({"bound": "hbm", "achieved": round(got, 1), "frac": round(got / PEAK_HBM_GBS, 4),
+                                  "frac_of_measured": round(got / peaks["read_GBs"], 4)})
+                else:
+                    point.update(hbm_roofline(cfg, elt, b, CONTEXT + w + (k + 1) / 2.0, ms, peaks))
+                if b == 8:
+                    def one_step():
+                        t = runner.decode_launch(ids, None, [0.0] * b, [0] * b, [1.0] * b, [0.0] * b,
+                                                 feed_rows=list(range(b)))
+                        runner.decode_collect(t)
+                    point["kernels"] = kernel_split(one_step, 4)
+                release(runner, ids)
+                rec[f"decode_b{b}"] = point
+            out[f"{design}_{tag}"] = rec
+            del runner
+            torch.cuda.empty_cache()
+    head = out["rupezen_w4096"]["decode_b8"]
+    return {"metric": "decode tok/s (Rupezen design, width 4096, 8 layer runs, random weights)", "value": head["tok_s"],
+            "unit": "tok/s", "n_gpus": 1, "steps": k, "warmup": w, "ms_per_step": head["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+            "config": {"model": "Rupezen and Qwen3 designs at equal sizes", "layer_runs": runs, "vocab": vocab,
+                       "sizes": sizes, "global_batch": 8, "seq_len": CONTEXT, "parallelism": "single GPU"},
+            "measured": peaks, "designs": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--workload", default="decode_8b",
                     choices=["decode_8b", "continuous_4b", "long_32b", "contexts_8b", "products_8b", "decode_4b",
-                             "decode_32b", "kofipel"],
+                             "decode_32b", "kofipel", "rupezen"],
                     help="decode_8b: the headline run; the others: the 4B and 32B shapes with their own "
                          "workloads (one JSON line each, other fields)")
     ap.add_argument("--gpus", type=int, default=1)
@@ -709,7 +845,7 @@ def main():
         return 1
     if args.workload != "decode_8b":
         print(json.dumps({"continuous_4b": continuous_4b, "long_32b": long_32b,
-                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel,
+                          "contexts_8b": contexts_8b, "products_8b": products_8b, "kofipel": kofipel, "rupezen": rupezen,
                           "decode_4b": lambda a: decode_shape(a, QWEN3_4B, "Qwen3-4B", 0.02),
                           "decode_32b": lambda a: decode_shape(a, QWEN3_32B, "Qwen3-32B", 0.01)}[args.workload](args)))
         return 0

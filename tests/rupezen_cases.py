@@ -37,7 +37,7 @@ RUPE_A_INIT = dict(seed=21, std=0.12, embedding_std=1.0, norm_jitter=0.1)
 
 # no loop; nothing a power of two; one layer with plain causal attention; groups of one expert; a factor of 1
 RUPE_B = {
-    "architecture": "Rupezen", "vocab": 97, "width": 72, "norm": {"eps": 3e-6}, "residual_mult": 1.0,
+    "architecture": "Rupezen", "vocab": 97, "width": 76, "norm": {"eps": 3e-6}, "residual_mult": 1.0,
     "layers": [
         _layer(3, 3, 10, 20, 0.3, 0.5, chunk=17, rot=(1000.0, 10), moe=(20, 6, 2, 6, 3)),
         _layer(6, 1, 6, 14, 0.4, 0.1, chunk=None, rot=(50.0, 2), moe=(28, 9, 4, 3, 2)),
