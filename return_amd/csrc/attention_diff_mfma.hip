@@ -1,5 +1,5 @@
-// Differential attention on the matrix cores, bfloat16: portions of prompts (two or more new tokens of a
-// request) over what the paged cache holds for them. The formulas, the masks (causal, window, chunk) and
+// Differential attention on the matrix cores, bfloat16: the new tokens of a request, a portion of a prompt or
+// a single token, over what the paged cache holds for it. The formulas, the masks (causal, window, chunk) and
 // the tables are those of attention_diff.hip; sizes: a map of D = 16, 32, 48, 64, 96 or 128 elements,
 // values of Dv = 32, 64, 96, 128, 192 or 256.
 //
@@ -44,7 +44,9 @@ __device__ __forceinline__ int diff_first_key(int p, int start, int window, int 
     return f;
 }
 
-template <int D16, int DV16, int BN>
+// PACK (tiles of one row: requests that bring one token): a workgroup takes a kv head and the rows of its first
+// wave are the query heads of that kv head's group (up to 16), so the group's keys and values are read once.
+template <int D16, int DV16, int BN, bool PACK>
 __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* __restrict__ k_pool,
     const bf16* __restrict__ v_pool, const int* __restrict__ page_table,
@@ -52,7 +54,7 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     const int* __restrict__ tiles,       // [n_tiles][2]: request number, first row of the tile within it
     int n_tiles, int Hq, int Hkv, int P, float scale, int window, int chunk, float lambda, float eps,
-    float out_scale) {
+    float out_scale, int n_splits, float* __restrict__ part) {
     constexpr int D = 16 * D16, DK = 2 * D, DV = 16 * DV16;
     constexpr int D32 = D / 32;
     constexpr bool TAIL16 = (D % 32) != 0;
@@ -63,18 +65,20 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     __shared__ __attribute__((aligned(16))) uint16_t k_s[BN * KS];
     __shared__ __attribute__((aligned(16))) uint16_t v_s[BN * VS];
 
-    const int head = blockIdx.x % Hq, tile = blockIdx.x / Hq;
-    const int seg = tiles[2 * tile], q_off = tiles[2 * tile + 1];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
-    const int kvh = head / (Hq / Hkv);
+    const int grp = Hq / Hkv;
+    const int tile = PACK ? blockIdx.x / Hkv : blockIdx.x / Hq;
+    const int kvh = PACK ? blockIdx.x % Hkv : (blockIdx.x % Hq) / grp;
+    const int head = PACK ? kvh * grp + min(n, grp - 1) : blockIdx.x % Hq;     // (PACK: this lane's row is a head of its own)
+    const int seg = tiles[2 * tile], q_off = tiles[2 * tile + 1];
     const int q_len = cu_q[seg + 1] - cu_q[seg];
     const int pos0 = q_start[seg];
     const int start = kv_start[seg];
     const int* pt = page_table + cu_pages[seg];
 
     // this lane's query row (for the B operands and for the mask): row n of the wave's 16
-    const int q_local = q_off + wave * 16 + n;
-    const bool q_ok = q_local < q_len;
+    const int q_local = PACK ? q_off : q_off + wave * 16 + n;
+    const bool q_ok = PACK ? (wave == 0 && n < grp && q_local < q_len) : q_local < q_len;
     const int pos_q = pos0 + q_local;
     const int first_q = diff_first_key(pos_q, start, window, chunk);
     const dbf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -100,7 +104,7 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     const int low_key = diff_first_key(tile_first_pos, start, window, chunk);    // the earliest key any row reads
     const int u_first = (low_key / BN) * BN;
     // the wave's rows: positions, and the first keys of its first and last row (first keys rise with the position)
-    const int wave_first_pos = tile_first_pos + wave * 16, wave_last_pos = wave_first_pos + 15;
+    const int wave_first_pos = tile_first_pos + wave * 16, wave_last_pos = PACK ? wave_first_pos : wave_first_pos + 15;
     const int wave_low = diff_first_key(wave_first_pos, start, window, chunk);
     const int wave_high = diff_first_key(wave_last_pos, start, window, chunk);
 
@@ -155,15 +159,26 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
         }                                                                                 \
     }
 
-    DIFF_FETCH(u_first)
-    for (int u = u_first; u <= tile_last_pos; u += BN) {
+    // With n_splits > 1 (tiles of one row: requests that bring one token) the workgroups blockIdx.y = 0, 1, ...
+    // share the tile's key blocks evenly and leave their sums to the merge kernel.
+    int u_lo = u_first, u_hi = tile_last_pos;            // first key block, and the last key, of this workgroup
+    if (n_splits > 1) {
+        const int blocks = (tile_last_pos - u_first) / BN + 1;
+        const int per = (blocks + n_splits - 1) / n_splits;
+        u_lo = u_first + (int)blockIdx.y * per * BN;
+        u_hi = min(tile_last_pos, u_lo + per * BN - 1);
+    }
+    if (u_lo <= u_hi) DIFF_FETCH(u_lo)
+    for (int u = u_lo; u <= u_hi; u += BN) {
         __syncthreads();                                 // every wave is done with the tile before
         DIFF_STAGE()
         __syncthreads();
-        if (u + BN <= tile_last_pos) DIFF_FETCH(u + BN)  // on its way while this tile is used
+        if (u + BN <= u_hi) DIFF_FETCH(u + BN)           // on its way while this tile is used
 
-        // a tile that lies wholly above every row of the wave, or wholly before their first keys, has nothing for it
-        if (u <= wave_last_pos && u + BN - 1 >= wave_low) {
+        // a tile that lies wholly above every row of the wave, or wholly before their first keys, has nothing for
+        // it; nor has any tile for a wave whose rows all lie beyond the request's new tokens (a request that
+        // brings one token: three waves only help to move the tiles)
+        if (u <= wave_last_pos && u + BN - 1 >= wave_low && wave_first_pos <= tile_last_pos) {
             dfloat4_t cs[2][BN / 16];
 #pragma unroll
             for (int st = 0; st < BN / 16; ++st) {
@@ -278,6 +293,25 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
 #undef DIFF_STAGE
     MFMA_SETTLE();
     // ---- acc[mp][dt][i] = O^T[d = 16dt + 4g + i][query n]
+    if (n_splits > 1) {
+        // the tile's one row is lane n = 0 of wave 0: per map the running maximum (a raw score), the sum and
+        // the unnormed row
+        if (PACK ? q_ok : (wave == 0 && n == 0)) {
+            float* pp = part + (((size_t)tile * Hq + head) * n_splits + blockIdx.y) * 2 * (DV + 2);
+#pragma unroll
+            for (int mp = 0; mp < 2; ++mp) {
+                float* pm = pp + mp * (DV + 2);
+                if (g == 0) {
+                    pm[0] = m_run[mp];
+                    pm[1] = l_run[mp];
+                }
+#pragma unroll
+                for (int dt = 0; dt < DV16; ++dt)
+                    *reinterpret_cast<dfloat4_t*>(pm + 2 + dt * 16 + 4 * g) = acc[mp][dt];
+            }
+        }
+        return;
+    }
     const float inv1 = l_run[0] > 0.f ? 1.0f / l_run[0] : 0.f;
     const float inv2 = l_run[1] > 0.f ? lambda / l_run[1] : 0.f;
     float ss = 0.f;
@@ -306,14 +340,21 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
 #define DIFF_CAT(a, b) DIFF_CAT2(a, b)
 #define DIFF_PART_ARGS int DV16, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp, const bf16* vp,   \
     const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs, const int* tiles, int n_tiles, int Hq,  \
-    int Hkv, int P, float scale, int window, int chunk, float lambda, float eps, float out_scale
+    int Hkv, int P, float scale, int window, int chunk, float lambda, float eps, float out_scale, int n_splits, float* part, \
+    int pack
 extern "C" int DIFF_CAT(ra_diff_part_, DIFF_D16)(DIFF_PART_ARGS) {
     // 64 keys a pass while a tile of them fits 40 KB of LDS, else 32
 #define DIFF_CASE(V_)                                                                                           \
     case V_: {                                                                                                  \
         constexpr int BN_ = (64 * (2 * 16 * DIFF_D16 + 8 + 16 * V_ + 16) * 2 <= 40960) ? 64 : 32;               \
-        hipLaunchKernelGGL((attn_diff_mfma_kernel<DIFF_D16, V_, BN_>), grid, dim3(256), 0, st, q, out, kp, vp, pt, cup, \
-                           kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window, chunk, lambda, eps, out_scale); \
+        if (pack)                                                                                               \
+            hipLaunchKernelGGL((attn_diff_mfma_kernel<DIFF_D16, V_, BN_, true>), grid, dim3(256), 0, st, q, out, kp, vp, pt, \
+                               cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window, chunk, lambda, eps,  \
+                               out_scale, n_splits, part);                                                      \
+        else                                                                                                    \
+            hipLaunchKernelGGL((attn_diff_mfma_kernel<DIFF_D16, V_, BN_, false>), grid, dim3(256), 0, st, q, out, kp, vp, pt, \
+                               cup, kvs, cuq, qs, tiles, n_tiles, Hq, Hkv, P, scale, window, chunk, lambda, eps,  \
+                               out_scale, n_splits, part);                                                      \
         return RA_OK;                                                                                           \
     }
     switch (DV16) {
@@ -327,7 +368,8 @@ extern "C" int DIFF_CAT(ra_diff_part_, DIFF_D16)(DIFF_PART_ARGS) {
 #ifdef DIFF_API
 #define DIFF_PART_ARGS int DV16, dim3 grid, hipStream_t st, const bf16* q, bf16* out, const bf16* kp, const bf16* vp,   \
     const int* pt, const int* cup, const int* kvs, const int* cuq, const int* qs, const int* tiles, int n_tiles, int Hq,  \
-    int Hkv, int P, float scale, int window, int chunk, float lambda, float eps, float out_scale
+    int Hkv, int P, float scale, int window, int chunk, float lambda, float eps, float out_scale, int n_splits, float* part, \
+    int pack
 extern "C" int ra_diff_part_1(DIFF_PART_ARGS);
 extern "C" int ra_diff_part_2(DIFF_PART_ARGS);
 extern "C" int ra_diff_part_3(DIFF_PART_ARGS);
@@ -344,24 +386,73 @@ extern "C" int ra_attention_diff_mfma_fits(int D, int Dv) {
     return d_ok && v_ok;
 }
 
+// The sums of a one-row tile's splits into its output row: per map the splits' maxima, sums and unnormed rows
+// are merged in split order; then lambda, the head's norm and the factor. One wave per (tile, head).
+__global__ __launch_bounds__(64) void attn_diff_merge_kernel(const float* __restrict__ part, bf16* __restrict__ out,
+                                                             const int* __restrict__ tiles, const int* __restrict__ cu_q,
+                                                             int Hq, int DV, int n_splits, float scale, float lambda,
+                                                             float eps, float out_scale) {
+    const int tile = blockIdx.x / Hq, head = blockIdx.x % Hq, lane = threadIdx.x;
+    const float scale2 = scale * 1.44269504088896340736f;
+    const float* pp = part + (size_t)blockIdx.x * n_splits * 2 * (DV + 2);
+    float o[4] = {0.f, 0.f, 0.f, 0.f};                   // elements lane, lane + 64, ... (DV <= 256)
+#pragma unroll
+    for (int mp = 0; mp < 2; ++mp) {
+        float m = -INFINITY;
+        for (int sp = 0; sp < n_splits; ++sp) m = fmaxf(m, pp[(sp * 2 + mp) * (DV + 2)]);
+        float l = 0.f, a[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int sp = 0; sp < n_splits; ++sp) {
+            const float* pm = pp + (sp * 2 + mp) * (DV + 2);
+            if (pm[0] == -INFINITY) continue;            // a split that saw no key
+            const float wgt = __builtin_amdgcn_exp2f((pm[0] - m) * scale2);
+            l = fmaf(pm[1], wgt, l);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (lane + 64 * i < DV) a[i] = fmaf(pm[2 + lane + 64 * i], wgt, a[i]);
+        }
+        const float f = l > 0.f ? (mp == 0 ? 1.0f : -lambda) / l : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = fmaf(a[i], f, o[i]);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (lane + 64 * i < DV) ss = fmaf(o[i], o[i], ss);
+    ss = wave_sum(ss);
+    const float f = out_scale / sqrtf(ss / (float)DV + eps);
+    bf16* op = out + ((size_t)cu_q[tiles[2 * tile]] * Hq + head) * DV;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (lane + 64 * i < DV) op[lane + 64 * i] = from_f<bf16>(o[i] * f);
+}
+
+// floats of the buffer that n_splits > 1 needs for n_tiles one-row tiles
+extern "C" long long ra_attention_diff_mfma_part_floats(int n_tiles, int Hq, int Dv, int n_splits) {
+    return (long long)n_tiles * Hq * n_splits * 2 * (Dv + 2);
+}
+
 // tiles: int32 [n_tiles][2] = (request number, first row of the tile within the request's new tokens), tiles
-// of 64 rows over every request with more than one new token.
+// of 64 rows over the requests to work on (a request that brings one token is one tile with one row).
+// n_splits > 1: every tile has ONE row (requests that bring one token), its keys are shared among n_splits
+// workgroups whose sums go through part (ra_attention_diff_mfma_part_floats floats) and the merge kernel.
+// pack (one-row tiles, at most 16 query heads a kv head): a workgroup per kv head works on all heads of its group.
 extern "C" int ra_attention_diff_mfma_bf16(const void* q, void* out, const void* k_pool, const void* v_pool,
                                            const int* page_table, const int* cu_pages, const int* kv_start,
                                            const int* cu_q, const int* q_start, const int* tiles, int n_tiles,
                                            int Hq, int Hkv, int D, int Dv, int P, float scale, int window, int chunk,
-                                           float lambda, float eps, float out_scale, void* stream) {
+                                           float lambda, float eps, float out_scale, int n_splits, float* part,
+                                           int pack, void* stream) {
     if (n_tiles <= 0) return RA_OK;
-    if (!ra_attention_diff_mfma_fits(D, Dv) || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 ||
-        (long long)n_tiles * Hq > 0x7fffffffLL)
+    if (!ra_attention_diff_mfma_fits(D, Dv) || Hkv <= 0 || Hq % Hkv != 0 || P <= 0 || n_splits < 1 || n_splits > 65535 ||
+        (n_splits > 1 && part == nullptr) || (long long)n_tiles * Hq > 0x7fffffffLL || (pack && Hq / Hkv > 16))
         return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
-    dim3 grid(n_tiles * Hq);
+    dim3 grid(n_tiles * (pack ? Hkv : Hq), n_splits);
     int rc;
 #define DIFF_GO(k)                                                                                            \
     rc = ra_diff_part_##k(Dv / 16, grid, st, (const bf16*)q, (bf16*)out, (const bf16*)k_pool, (const bf16*)v_pool, \
                           page_table, cu_pages, kv_start, cu_q, q_start, tiles, n_tiles, Hq, Hkv, P, scale, window, \
-                          chunk, lambda, eps, out_scale)
+                          chunk, lambda, eps, out_scale, n_splits, part, pack)
     switch (D / 16) {
         case 1: DIFF_GO(1); break;
         case 2: DIFF_GO(2); break;
@@ -373,6 +464,9 @@ extern "C" int ra_attention_diff_mfma_bf16(const void* q, void* out, const void*
     }
 #undef DIFF_GO
     if (rc != RA_OK) return rc;
+    if (n_splits > 1)
+        hipLaunchKernelGGL(attn_diff_merge_kernel, dim3(n_tiles * Hq), dim3(64), 0, st, part, (bf16*)out, tiles, cu_q, Hq,
+                           Dv, n_splits, scale, lambda, eps, out_scale);
     return ra_launch_status();
 }
 #endif  // DIFF_API

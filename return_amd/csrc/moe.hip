@@ -12,7 +12,9 @@
 //             One workgroup (a counting sort). A pair's result does not depend on its place in a tile.
 //   product   for every tile: y[p] = W_e x[row(p)] with row(p) = p / top (the token's row) or p itself;
 //             gated: W_e = [gate rows; up rows], y = silu(gate) * up. An FMA form for every size and both
-//             storage types, and a matrix-core form for bfloat16 with K % 8 == 0.
+//             storage types, and two matrix-core forms for bfloat16 with K % 8 == 0: operands straight from
+//             memory for tiles of 16 or 64 rows (few rows an expert: the weights are read once, the time is
+//             the reading), tiles of 128 rows staged in LDS where an expert has many rows.
 //   combine   out[t] = sum_k weights[t][k] * y[t * top + k], k in order, 32-bit sums.
 #include "common.h"
 
@@ -296,9 +298,129 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(
     }
 }
 
+// ------------------------------------------------------------------ product, matrix-core form with tiles in LDS
+// For many rows per expert: a workgroup per (tile of up to 128 rows of one expert, 128 result columns, or 64
+// gated ones with their gate and up rows), k-steps of 32, four waves as 2 x 2, each 64 x 64 as 4 x 4 MFMA tiles;
+// both operands staged in LDS with padded rows, two buffers, the next k-step travelling through registers (the
+// scheme of the tiled product for many rows, with the rows of x gathered by pair and W taken from the expert).
+// Gated: of a wave's four tiles of W rows the first two are gate rows and the last two the up rows of the same
+// columns, so a lane holds both halves of a result and forms silu(gate) * up itself.
+#define MT_BM 128
+#define MT_BK 32
+#define MT_LD (MT_BK + 8)
+typedef uint32_t moe_uint4_t __attribute__((ext_vector_type(4)));
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_product_tile_kernel(
+    const bf16* __restrict__ x, const bf16* __restrict__ w, bf16* __restrict__ y, const int* __restrict__ order,
+    const int* __restrict__ tiles, const int* __restrict__ meta, int N, int K, int top_div) {
+    if ((int)blockIdx.x >= meta[0]) return;
+    __shared__ __attribute__((aligned(16))) uint16_t a_s[2][MT_BM * MT_LD];
+    __shared__ __attribute__((aligned(16))) uint16_t w_s[2][128 * MT_LD];
+    constexpr int CN = GATED ? 64 : 128;                       // result columns per workgroup
+    const int e = tiles[3 * blockIdx.x], at = tiles[3 * blockIdx.x + 1], n_rows = tiles[3 * blockIdx.x + 2];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 15, g = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int n0 = blockIdx.y * CN;
+
+    // staging: 128 rows x 4 pieces of 16 bytes per operand; a thread moves 2 pieces of each
+    const int ld_row = tid >> 1, ld_p = (tid & 1) * 2;
+    const int a_pair = order[at + min(ld_row, n_rows - 1)];
+    const bf16* a_src = x + (size_t)(a_pair / top_div) * K + ld_p * 8;
+    size_t w_row;
+    if (GATED) {
+        const int t4 = (ld_row >> 4) & 3;                      // which of the wave's four tiles of W rows
+        const int col = n0 + (ld_row >> 6) * 32 + (t4 & 1) * 16 + (ld_row & 15);
+        w_row = (size_t)e * 2 * N + (size_t)(t4 >> 1) * N + min(col, N - 1);
+    } else {
+        w_row = (size_t)e * N + min(n0 + ld_row, N - 1);
+    }
+    const bf16* w_src = w + w_row * K + ld_p * 8;
+    const moe_uint4_t zero = {0u, 0u, 0u, 0u};
+    moe_uint4_t ar[2], wr[2];
+    moe_float4_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = moe_float4_t{0.f, 0.f, 0.f, 0.f};
+#define MT_FETCH(k0_)                                                                        \
+    _Pragma("unroll") for (int p = 0; p < 2; ++p) {                                          \
+        const bool in_ = (k0_) + (ld_p + p) * 8 < K;                                         \
+        ar[p] = in_ ? *reinterpret_cast<const moe_uint4_t*>(a_src + (k0_) + p * 8) : zero;   \
+        wr[p] = in_ ? *reinterpret_cast<const moe_uint4_t*>(w_src + (k0_) + p * 8) : zero;   \
+    }
+#define MT_STAGE(buf_)                                                                       \
+    _Pragma("unroll") for (int p = 0; p < 2; ++p) {                                          \
+        *reinterpret_cast<moe_uint4_t*>(&a_s[buf_][ld_row * MT_LD + (ld_p + p) * 8]) = ar[p]; \
+        *reinterpret_cast<moe_uint4_t*>(&w_s[buf_][ld_row * MT_LD + (ld_p + p) * 8]) = wr[p]; \
+    }
+    MT_FETCH(0)
+    MT_STAGE(0)
+    if (MT_BK < K) { MT_FETCH(MT_BK) }
+    __syncthreads();
+    const bool rows_here = wm * 64 < n_rows;                  // (a wave whose rows all lie beyond the tile's only moves data)
+    int it = 0;
+    for (int k0 = 0; k0 < K; k0 += MT_BK, ++it) {
+        const int cur = it & 1;
+        if (k0 + MT_BK < K) {
+            MT_STAGE(cur ^ 1)
+            if (k0 + 2 * MT_BK < K) { MT_FETCH(k0 + 2 * MT_BK) }
+        }
+        if (rows_here) {
+            moe_bf16x8_t af[4], wf[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                af[i] = *reinterpret_cast<const moe_bf16x8_t*>(&a_s[cur][(wm * 64 + i * 16 + n) * MT_LD + 8 * g]);
+                wf[i] = *reinterpret_cast<const moe_bf16x8_t*>(&w_s[cur][(wn * 64 + i * 16 + n) * MT_LD + 8 * g]);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (wm * 64 + j * 16 >= n_rows) break;         // (the same in every lane: groups of rows beyond the tile's)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], af[j], acc[i][j], 0, 0, 0);
+            }
+        }
+        __syncthreads();
+    }
+#undef MT_FETCH
+#undef MT_STAGE
+    MFMA_SETTLE();
+    // acc[i][j][e]: row wm*64 + j*16 + n of the tile, W row (wn*64 + i*16 + 4g + e) of the workgroup's 128
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int m = wm * 64 + j * 16 + n;
+        if (m >= n_rows) continue;
+        bf16* yr = y + (size_t)order[at + m] * N;
+#pragma unroll
+        for (int i = 0; i < (GATED ? 2 : 4); ++i) {
+            const int col = GATED ? n0 + wn * 32 + i * 16 + 4 * g : n0 + wn * 64 + i * 16 + 4 * g;
+            float v[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                v[c] = acc[i][j][c];
+                if (GATED) {
+                    const float gg = round_to<bf16>(acc[i][j][c]), uu = round_to<bf16>(acc[i + 2][j][c]);
+                    v[c] = gg / (1.0f + expf(-gg)) * uu;
+                }
+            }
+            if (col + 3 < N && (N & 3) == 0) {
+                uint2 pk;
+                pk.x = (uint32_t)f2bf_bits(v[0]) | ((uint32_t)f2bf_bits(v[1]) << 16);
+                pk.y = (uint32_t)f2bf_bits(v[2]) | ((uint32_t)f2bf_bits(v[3]) << 16);
+                *reinterpret_cast<uint2*>(yr + col) = pk;
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; ++c)
+                    if (col + c < N) yr[col + c] = from_f<bf16>(v[c]);
+            }
+        }
+    }
+}
+
 // rows of a tile that the product kernel behind these arguments takes (what ra_moe_plan is to be called with)
 extern "C" int ra_moe_tile_rows(int n_pairs, int E, int K, int dtype) {
-    if (dtype == RA_DTYPE_BF16 && K % 8 == 0) return n_pairs >= 24 * E ? 64 : 16;
+    if (dtype == RA_DTYPE_BF16 && K % 8 == 0) return n_pairs >= 64 * E ? 128 : (n_pairs >= 24 * E ? 64 : 16);
     return MOE_FMA_ROWS;
 }
 
@@ -311,6 +433,18 @@ extern "C" int ra_moe_product(const void* x, const void* w, void* y, const int* 
     if (max_tiles <= 0) return RA_OK;
     if (N < 1 || K < 1 || top_div < 1) return RA_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
+    if (dtype == RA_DTYPE_BF16 && K % 8 == 0 && tile_rows == MT_BM) {
+        const int cn = gated ? 64 : 128;
+        dim3 grid(max_tiles, (N + cn - 1) / cn);
+        if (grid.y > 65535) return RA_ERR_ARG;
+        if (gated)
+            hipLaunchKernelGGL(moe_product_tile_kernel<true>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w,
+                               (bf16*)y, order, tiles, meta, N, K, top_div);
+        else
+            hipLaunchKernelGGL(moe_product_tile_kernel<false>, grid, dim3(256), 0, st, (const bf16*)x, (const bf16*)w,
+                               (bf16*)y, order, tiles, meta, N, K, top_div);
+        return ra_launch_status();
+    }
     if (dtype == RA_DTYPE_BF16 && K % 8 == 0 && (tile_rows == 16 || tile_rows == 64)) {
         const bf16 *xb = (const bf16*)x, *wb = (const bf16*)w;
         bf16* yb = (bf16*)y;

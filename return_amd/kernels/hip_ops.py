@@ -56,7 +56,7 @@ def _declare(lib):
         "ra_stream_pair_rows": [P, P, F, P, P, L, I, I, P],
         "ra_maps_qkv_prepare": [P, I, I, I, I, I, I, P, P, P, I, I, P, P, P, P, I, I, P],
         "ra_attention_diff_plain": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, F, I, I, F, F, F, I, P],
-        "ra_attention_diff_mfma_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, F, F, F, P],
+        "ra_attention_diff_mfma_bf16": [P, P, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, I, F, F, F, I, P, I, P],
         "ra_attention_diff_mfma_fits": [I, I],
         "ra_attention_diff_plain_fits": [I, I],
         "ra_moe_route": [P, P, I, I, I, I, I, F, P, P, P],
@@ -161,10 +161,16 @@ class HipOps:
         want = a.double() @ b.double().t()
         self._library_fp32_exact = bool(((torch.matmul(a, b.t()).double() - want).abs().max()
                                          <= 2e-5 * want.abs().max()).item())
+        self._unit_tiles = self._make_unit_tiles(1024)    # (i, 0) for i = 0, 1, ...: q tiles of requests that bring one token each
         self.product_plan = {}               # (row step, N, K, gated, result dtype) -> way, where measured faster than the rule
         self._measured = _PRODUCTS_MEASURED
         self._times = _PRODUCT_TIMES
         self._defer = {}                     # as _NORM_PAIRS_MEASURED, for the pairs this kernel set has been shown
+
+    def _make_unit_tiles(self, n):
+        t = torch.zeros(n, 2, dtype=torch.int32, device=self.device)
+        t[:, 0] = torch.arange(n, dtype=torch.int32, device=self.device)
+        return t
 
     def use_skinny(self, M, N, K, out_dtype):
         """Whether the hand-written skinny product beats the library for x [M, K] @ W[N, K]^T
@@ -1259,18 +1265,50 @@ class HipOps:
                 step.n_seqs, rows, n_q, n_kv, D2 // 2, Dv, P, *consts, _code(q.dtype), self._stream()),
                 "attention_diff_plain")
 
-        tiles = step.prefill_tiles.get(64) if getattr(step, "prefill_tiles", None) else None
-        if tiles is not None and step.n_prefill_tokens > 0 and q.dtype == torch.bfloat16 and scale > 0 and \
-                self.lib.ra_attention_diff_mfma_fits(D2 // 2, Dv):
-            # requests with two or more new tokens on the matrix cores, tile by tile; the others (one token
-            # each) by the plain kernel, a workgroup of eight waves over the keys of each
-            self._check(self.lib.ra_attention_diff_mfma_bf16(
-                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], n_q, n_kv,
-                D2 // 2, Dv, P, *consts, self._stream()), "attention_diff_mfma_bf16")
+        if q.dtype == torch.bfloat16 and scale > 0 and self.lib.ra_attention_diff_mfma_fits(D2 // 2, Dv):
+            # the matrix-core kernel, tile by tile: the q tiles of the requests with two or more new tokens, and
+            # one tile of one row for every request that brings a single token
+            lists = []
+            if step.n_prefill_tokens > 0:
+                tiles = step.prefill_tiles.get(64) if getattr(step, "prefill_tiles", None) else None
+                if tiles is None:
+                    raise KernelError("attention_diff: the step lists no q tiles of 64 rows")
+                lists.append((tiles, 1, 0))
             if step.n_decode > 0:
-                plain(step.decode_segs, True, step.n_decode)
+                if step.decode_segs is None:             # every request brings one token: request i is tile (i, 0)
+                    if step.n_decode > self._unit_tiles.shape[0]:
+                        self._unit_tiles = self._make_unit_tiles(2 * step.n_decode)
+                    tiles = self._unit_tiles[:step.n_decode]
+                else:
+                    tiles = torch.stack([step.decode_segs, torch.zeros_like(step.decode_segs)], dim=1).contiguous()
+                # (one kv head's group of query heads as the rows of one workgroup, where it fits a tile of rows)
+                pack = 1 if n_q // n_kv <= 16 else 0
+                lists.append((tiles, self._diff_decode_splits(step, n_kv if pack else n_q, int(window), int(chunk)), pack))
+            for tiles, splits, pack in lists:
+                part = None
+                if splits > 1:
+                    part = torch.empty(tiles.shape[0] * n_q * splits * 2 * (Dv + 2), dtype=torch.float32, device=self.device)
+                self._check(self.lib.ra_attention_diff_mfma_bf16(
+                    _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], n_q, n_kv,
+                    D2 // 2, Dv, P, *consts, splits, _ptr(part), pack, self._stream()), "attention_diff_mfma_bf16")
             return
         plain(None, False, T)
+
+    def _diff_decode_splits(self, step, n_heads, window, chunk):
+        """Workgroups that share the keys of a request that brings one token: enough of them to fill the chip
+        (about eight a CU), at least four blocks of 64 keys each. Decided by the step's class (the batch size and
+        context bucket of the graph that serves or would serve it) where the runner names one, so that a step run
+        eagerly and its replay from a graph sum in the same order."""
+        rule = getattr(step, "decode_rule", None)
+        n, longest = rule if rule else (step.n_decode, getattr(step, "max_decode_seq_len", 0))
+        keys = longest
+        if window > 0:
+            keys = min(keys, window)
+        if chunk > 0:
+            keys = min(keys, chunk)
+        blocks = -(-max(int(keys), 1) // 64)
+        want = -(-8 * self.cu_count // max(1, n * n_heads))
+        return int(max(1, min(64, want, blocks // 4)))
 
     # ------------------------------------------------------------------ routed experts
     MAX_EXPERTS = 1024

@@ -134,7 +134,8 @@ def run_attention_in_pieces(ops, h, w, m, eps, pieces, P=16, pages=(2, 0, 3, 1),
         tiles = {} if n == 1 else {64: i32([[0, off] for off in range(0, n, 64)])}      # q tiles, for a kernel that reads them
         step = types.SimpleNamespace(groups=[grp], n_seqs=1, n_tokens=n, cu_q=i32([0, n]), q_start=i32([at]),
                                      n_decode=1 if n == 1 else 0, prefill_tiles=tiles, q_lens=[n], q_starts=[at],
-                                     n_prefill_tokens=0 if n == 1 else n, decode_segs=None, prefill_toks=None)
+                                     n_prefill_tokens=0 if n == 1 else n, decode_segs=None, prefill_toks=None,
+                                     max_decode_seq_len=at + n if n == 1 else 0)
         q = torch.empty(n, H, 2 * D, dtype=dtype, device=device)
         ops.maps_qkv_prepare(qkv[at:at + n].contiguous(), H, G, 2, D, V, i32(pos), cos, sin, R, True, q, kp, vp, slots)
         o = torch.empty(n, H, V, dtype=dtype, device=device)

@@ -129,6 +129,29 @@ def test_attention_in_pieces_equals_the_plain_function(ops, ref, dtype, sizes, p
         assert float(err.max()) < 0.2 and float(err.mean()) < 0.02, f"row {int(err.argmax())}: {float(err.max()):.3e}"
 
 
+@pytest.mark.parametrize("sizes", [(2, 1, 64, 128, None, 16), (4, 2, 32, 64, 500, 32), (1, 1, 16, 32, 1100, 0)])
+def test_single_tokens_over_a_long_context(ops, ref, sizes):
+    """A long prompt and then tokens one by one: the matrix-core kernel shares a request's keys among several
+    workgroups and merges their sums (more than a thousand keys, with and without a chunk border on the way)."""
+    H, G, D, V, chunk, R = sizes
+    g = torch.Generator().manual_seed(D)
+    pieces = (1190, *([1] * 24))
+    T, W = sum(pieces), 24
+    m = {"heads": H, "kv_heads": G, "dim": D, "vdim": V, "scale": 2.0 / D, "diff": 0.35}
+    if chunk:
+        m["mask"] = {"size": chunk}
+    if R:
+        m["rot"] = {"base": 100.0, "dims": R}
+    w = {k: v.bfloat16().double() for k, v in _attention_weights(g, W, H, G, D, V).items()}
+    h = torch.randn(T, W, generator=g).bfloat16().double()
+    pages = tuple(torch.randperm(80, generator=g).tolist())
+    got = run_attention_in_pieces(ops, h, w, m, 1e-5, pieces, pages=pages, dtype=torch.bfloat16, device=DEV)
+    alike = run_attention_in_pieces(ref, h, w, m, 1e-5, pieces, pages=pages, dtype=torch.bfloat16, device=DEV)
+    err = (got.double() - alike.double()).pow(2).mean(-1).sqrt()
+    assert float(err.max()) < 0.02, f"row {int(err.argmax())}: {float(err.max()):.3e} from the stand-in"
+    assert ops._diff_decode_splits(types.SimpleNamespace(n_decode=1, max_decode_seq_len=T), H, 0, chunk or 0) > 1
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("D,V,C", [(8, 8, 10), (16, 32, 32), (64, 128, 48), (48, 96, 64)])
 @pytest.mark.parametrize("pieces_of", ["prompt", "decoded"])
@@ -180,7 +203,8 @@ def test_router_kernel_equals_the_plain_choice(ops, T, E, top, count, keep):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,H,I,E,top", [(1, 64, 24, 8, 2), (9, 72, 20, 6, 3), (37, 64, 40, 5, 1), (300, 96, 64, 4, 2),
-                                        (700, 128, 32, 8, 2), (3, 50, 13, 7, 7), (64, 256, 100, 64, 6)])
+                                        (700, 128, 32, 8, 2), (3, 50, 13, 7, 7), (64, 256, 100, 64, 6),
+                                        (1000, 256, 200, 8, 3), (520, 72, 136, 2, 2)])
 def test_experts_kernels_equal_the_stand_in(ops, ref, dtype, T, H, I, E, top):
     x = rnd(T, H, dtype=dtype, seed=1)
     gate_up = rnd(E, 2 * I, H, dtype=dtype, seed=2, scale=H ** -0.5)
