@@ -46,6 +46,8 @@ __device__ __forceinline__ int diff_first_key(int p, int start, int window, int 
 
 // PACK (tiles of one row: requests that bring one token): a workgroup takes a kv head and the rows of its first
 // wave are the query heads of that kv head's group (up to 16), so the group's keys and values are read once.
+// (One wave a workgroup, eight such workgroups a CU, was measured and is not faster: 77 against 65 us a layer at
+// batch 8 over 2,048 keys.)
 template <int D16, int DV16, int BN, bool PACK>
 __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     const bf16* __restrict__ q, bf16* __restrict__ out, const bf16* __restrict__ k_pool,
@@ -61,7 +63,8 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
     constexpr int KS = DK + 8;                          // K tile row stride (elements): rows shift by 4 banks
     constexpr int VS = DV + 16;                         // V tile row stride: rows shift by 8 banks (transposing reads)
     constexpr int LPRK = DK / 8, LPRV = DV / 8;         // 16-byte pieces in one row
-    constexpr int NK = (BN * LPRK + 255) / 256, NV = (BN * LPRV + 255) / 256;     // pieces per thread per tile
+    constexpr int NT = 256;                             // threads of the workgroup
+    constexpr int NK = (BN * LPRK + NT - 1) / NT, NV = (BN * LPRV + NT - 1) / NT;     // pieces per thread per tile
     __shared__ __attribute__((aligned(16))) uint16_t k_s[BN * KS];
     __shared__ __attribute__((aligned(16))) uint16_t v_s[BN * VS];
 
@@ -127,14 +130,14 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
 #define DIFF_FETCH(u_)                                                                    \
     {                                                                                     \
         _Pragma("unroll") for (int i = 0; i < NK; ++i) {                                  \
-            const int pc = tid + 256 * i;                                                 \
+            const int pc = tid + NT * i;                                                  \
             if (pc < BN * LPRK) {                                                         \
                 const int r_ = pc / LPRK, c_ = pc - r_ * LPRK;                            \
                 kreg[i] = *reinterpret_cast<const duint4_t*>(k_pool + (size_t)row_of((u_) + r_) * DK + 8 * c_); \
             }                                                                             \
         }                                                                                 \
         _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                  \
-            const int pc = tid + 256 * i;                                                 \
+            const int pc = tid + NT * i;                                                  \
             if (pc < BN * LPRV) {                                                         \
                 const int r_ = pc / LPRV, c_ = pc - r_ * LPRV;                            \
                 vreg[i] = *reinterpret_cast<const duint4_t*>(v_pool + (size_t)row_of((u_) + r_) * DV + 8 * c_); \
@@ -144,14 +147,14 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
 #define DIFF_STAGE()                                                                      \
     {                                                                                     \
         _Pragma("unroll") for (int i = 0; i < NK; ++i) {                                  \
-            const int pc = tid + 256 * i;                                                 \
+            const int pc = tid + NT * i;                                                  \
             if (pc < BN * LPRK) {                                                         \
                 const int r_ = pc / LPRK, c_ = pc - r_ * LPRK;                            \
                 *reinterpret_cast<duint4_t*>(k_s + r_ * KS + 8 * c_) = kreg[i];           \
             }                                                                             \
         }                                                                                 \
         _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                  \
-            const int pc = tid + 256 * i;                                                 \
+            const int pc = tid + NT * i;                                                  \
             if (pc < BN * LPRV) {                                                         \
                 const int r_ = pc / LPRV, c_ = pc - r_ * LPRV;                            \
                 *reinterpret_cast<duint4_t*>(v_s + r_ * VS + 8 * c_) = vreg[i];           \
@@ -398,14 +401,18 @@ __global__ __launch_bounds__(64) void attn_diff_merge_kernel(const float* __rest
     float o[4] = {0.f, 0.f, 0.f, 0.f};                   // elements lane, lane + 64, ... (DV <= 256)
 #pragma unroll
     for (int mp = 0; mp < 2; ++mp) {
-        float m = -INFINITY;
-        for (int sp = 0; sp < n_splits; ++sp) m = fmaxf(m, pp[(sp * 2 + mp) * (DV + 2)]);
+        // lane sp reads split sp's maximum and sum (n_splits <= 64), all at once; the weights go round by lane reads
+        const float* mine = pp + ((size_t)min(lane, n_splits - 1) * 2 + mp) * (DV + 2);
+        const float my_m = lane < n_splits ? mine[0] : -INFINITY;
+        const float my_l = lane < n_splits ? mine[1] : 0.f;
+        const float m = wave_max(my_m);
+        const float my_w = (my_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((my_m - m) * scale2);
         float l = 0.f, a[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int sp = 0; sp < n_splits; ++sp) {
-            const float* pm = pp + (sp * 2 + mp) * (DV + 2);
-            if (pm[0] == -INFINITY) continue;            // a split that saw no key
-            const float wgt = __builtin_amdgcn_exp2f((pm[0] - m) * scale2);
-            l = fmaf(pm[1], wgt, l);
+#pragma unroll 4
+        for (int sp = 0; sp < n_splits; ++sp) {          // in split order
+            const float wgt = __shfl(my_w, sp, 64);
+            l = fmaf(__shfl(my_l, sp, 64), wgt, l);
+            const float* pm = pp + ((size_t)sp * 2 + mp) * (DV + 2);
 #pragma unroll
             for (int i = 0; i < 4; ++i)
                 if (lane + 64 * i < DV) a[i] = fmaf(pm[2 + lane + 64 * i], wgt, a[i]);
