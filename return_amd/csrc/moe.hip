@@ -246,25 +246,34 @@ __global__ __launch_bounds__(256) void moe_product_mfma_kernel(
             au[r][c] = moe_float4_t{0.f, 0.f, 0.f, 0.f};
         }
     const moe_bf16x8_t z8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        const int k = k0 + 8 * g;
-        const bool in = k < K;                             // (K % 8 == 0: a group of 8 lies inside or outside)
-        moe_bf16x8_t b[RT], a[CT], a2[CT];
+    // several k-steps of 32 at a time (eight with tiles of 16 rows, four with 64), all their loads asked for before
+    // the first product: with one or two rows an expert the kernel only reads W, and a lane then has 128 (gated: 256)
+    // bytes of it on their way instead of 16
+    constexpr int KU = RT == 1 ? 8 : 4;
+    for (int k0 = 0; k0 < K; k0 += 32 * KU) {
+        moe_bf16x8_t b[KU][RT], a[KU][CT], a2[KU][CT];
 #pragma unroll
-        for (int r = 0; r < RT; ++r)
-            b[r] = (in && pair[r] >= 0) ? *reinterpret_cast<const moe_bf16x8_t*>(xr[r] + k) : z8;
-#pragma unroll
-        for (int c = 0; c < CT; ++c) {
-            a[c] = in ? *reinterpret_cast<const moe_bf16x8_t*>(wr[c] + k) : z8;
-            if (GATED) a2[c] = in ? *reinterpret_cast<const moe_bf16x8_t*>(wr[c] + (size_t)N * K + k) : z8;
-        }
-#pragma unroll
-        for (int r = 0; r < RT; ++r)
+        for (int u = 0; u < KU; ++u) {
+            const int k = k0 + 32 * u + 8 * g;
+            const bool in = k < K;                         // (K % 8 == 0: a group of 8 lies inside or outside)
 #pragma unroll
             for (int c = 0; c < CT; ++c) {
-                ag[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[c], b[r], ag[r][c], 0, 0, 0);
-                if (GATED) au[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[c], b[r], au[r][c], 0, 0, 0);
+                a[u][c] = in ? *reinterpret_cast<const moe_bf16x8_t*>(wr[c] + k) : z8;
+                if (GATED) a2[u][c] = in ? *reinterpret_cast<const moe_bf16x8_t*>(wr[c] + (size_t)N * K + k) : z8;
             }
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+                b[u][r] = (in && pair[r] >= 0) ? *reinterpret_cast<const moe_bf16x8_t*>(xr[r] + k) : z8;
+        }
+#pragma unroll
+        for (int u = 0; u < KU; ++u)
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+#pragma unroll
+                for (int c = 0; c < CT; ++c) {
+                    ag[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], b[u][r], ag[r][c], 0, 0, 0);
+                    if (GATED) au[r][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a2[u][c], b[u][r], au[r][c], 0, 0, 0);
+                }
     }
     MFMA_SETTLE();
     // ag[r][c][i] = result[row n of group r][column col0 + 16c + 4g + i]

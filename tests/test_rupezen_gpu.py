@@ -96,7 +96,7 @@ def test_maps_prepare(ops, ref, dtype, Hq, Hkv, D, Dv, R, inter):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("sizes", [(4, 2, 8, 24, 20, 4), (3, 3, 6, 7, None, 6), (2, 1, 10, 32, 16, 0), (2, 2, 16, 32, 33, 8),
-                                   (4, 1, 32, 48, 64, 32), (2, 1, 64, 128, 100, 16), (1, 1, 128, 64, 7, 64), (2, 2, 48, 96, 64, 12)])
+                                   (4, 1, 32, 48, 64, 32), (2, 1, 64, 128, 100, 16), (1, 1, 128, 64, 7, 64), (2, 2, 48, 96, 80, 24)])
 @pytest.mark.parametrize("pieces", [(150,), (118, *([1] * 32)), (7, 2, 24, 3, 64, 2, 5, 33, 9, 1)])
 def test_attention_in_pieces_equals_the_plain_function(ops, ref, dtype, sizes, pieces):
     H, G, D, V, chunk, R = sizes
@@ -153,7 +153,7 @@ def test_single_tokens_over_a_long_context(ops, ref, sizes):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("D,V,C", [(8, 8, 10), (16, 32, 32), (64, 128, 48), (48, 96, 64)])
+@pytest.mark.parametrize("D,V,C", [(8, 8, 10), (16, 32, 32), (64, 128, 48), (48, 96, 80)])
 @pytest.mark.parametrize("pieces_of", ["prompt", "decoded"])
 def test_one_key_decides_at_the_chunk_borders(ops, dtype, D, V, C, pieces_of):
     """Two keys with large values sit on the first and on the last place of a chunk (a page's first and last
