@@ -127,21 +127,31 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
         const int pi = p_shift >= 0 ? (idx >> p_shift) : (idx / P);
         return (pt[pi] * Hkv + kvh) * P + (idx - pi * P);
     };
-#define DIFF_FETCH(u_)                                                                    \
+    // The cache rows of a tile's pieces are looked up one pass before the pieces are asked for, so that a fetch
+    // does not wait for the page table first (a read that waits for a read costs more than a pass's products).
+    int rk[NK], rv[NV];
+#define DIFF_ROWS(u_)                                                                     \
     {                                                                                     \
         _Pragma("unroll") for (int i = 0; i < NK; ++i) {                                  \
             const int pc = tid + NT * i;                                                  \
-            if (pc < BN * LPRK) {                                                         \
-                const int r_ = pc / LPRK, c_ = pc - r_ * LPRK;                            \
-                kreg[i] = *reinterpret_cast<const duint4_t*>(k_pool + (size_t)row_of((u_) + r_) * DK + 8 * c_); \
-            }                                                                             \
+            rk[i] = pc < BN * LPRK ? row_of((u_) + pc / LPRK) : 0;                        \
         }                                                                                 \
         _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                  \
             const int pc = tid + NT * i;                                                  \
-            if (pc < BN * LPRV) {                                                         \
-                const int r_ = pc / LPRV, c_ = pc - r_ * LPRV;                            \
-                vreg[i] = *reinterpret_cast<const duint4_t*>(v_pool + (size_t)row_of((u_) + r_) * DV + 8 * c_); \
-            }                                                                             \
+            rv[i] = pc < BN * LPRV ? row_of((u_) + pc / LPRV) : 0;                        \
+        }                                                                                 \
+    }
+#define DIFF_FETCH()                                                                      \
+    {                                                                                     \
+        _Pragma("unroll") for (int i = 0; i < NK; ++i) {                                  \
+            const int pc = tid + NT * i;                                                  \
+            if (pc < BN * LPRK)                                                           \
+                kreg[i] = *reinterpret_cast<const duint4_t*>(k_pool + (size_t)rk[i] * DK + 8 * (pc % LPRK)); \
+        }                                                                                 \
+        _Pragma("unroll") for (int i = 0; i < NV; ++i) {                                  \
+            const int pc = tid + NT * i;                                                  \
+            if (pc < BN * LPRV)                                                           \
+                vreg[i] = *reinterpret_cast<const duint4_t*>(v_pool + (size_t)rv[i] * DV + 8 * (pc % LPRV)); \
         }                                                                                 \
     }
 #define DIFF_STAGE()                                                                      \
@@ -171,12 +181,19 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
         u_lo = u_first + (int)blockIdx.y * per * BN;
         u_hi = min(tile_last_pos, u_lo + per * BN - 1);
     }
-    if (u_lo <= u_hi) DIFF_FETCH(u_lo)
+    if (u_lo <= u_hi) {
+        DIFF_ROWS(u_lo)
+        DIFF_FETCH()
+        DIFF_ROWS(u_lo + BN)                             // (beyond the last key the rows are clamped to valid ones)
+    }
     for (int u = u_lo; u <= u_hi; u += BN) {
         __syncthreads();                                 // every wave is done with the tile before
         DIFF_STAGE()
         __syncthreads();
-        if (u + BN <= u_hi) DIFF_FETCH(u + BN)           // on its way while this tile is used
+        if (u + BN <= u_hi) {                            // the next tile, on its way while this one is used
+            DIFF_FETCH()
+            DIFF_ROWS(u + 2 * BN)
+        }
 
         // a tile that lies wholly above every row of the wave, or wholly before their first keys, has nothing for
         // it; nor has any tile for a wave whose rows all lie beyond the request's new tokens (a request that
@@ -293,6 +310,7 @@ __global__ __launch_bounds__(256) void attn_diff_mfma_kernel(
         }
     }
 #undef DIFF_FETCH
+#undef DIFF_ROWS
 #undef DIFF_STAGE
     MFMA_SETTLE();
     // ---- acc[mp][dt][i] = O^T[d = 16dt + 4g + i][query n]
@@ -399,27 +417,48 @@ __global__ __launch_bounds__(64) void attn_diff_merge_kernel(const float* __rest
     const float scale2 = scale * 1.44269504088896340736f;
     const float* pp = part + (size_t)blockIdx.x * n_splits * 2 * (DV + 2);
     float o[4] = {0.f, 0.f, 0.f, 0.f};                   // elements lane, lane + 64, ... (DV <= 256)
+    const int token_row = cu_q[tiles[2 * tile]];         // (asked for now: a read that waits for a read is the time here)
+    // lane sp reads split sp's maximum and sum of both maps (n_splits <= 64), all at once
+    float my_m[2], my_l[2];
 #pragma unroll
     for (int mp = 0; mp < 2; ++mp) {
-        // lane sp reads split sp's maximum and sum (n_splits <= 64), all at once; the weights go round by lane reads
         const float* mine = pp + ((size_t)min(lane, n_splits - 1) * 2 + mp) * (DV + 2);
-        const float my_m = lane < n_splits ? mine[0] : -INFINITY;
-        const float my_l = lane < n_splits ? mine[1] : 0.f;
-        const float m = wave_max(my_m);
-        const float my_w = (my_m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((my_m - m) * scale2);
-        float l = 0.f, a[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-        for (int sp = 0; sp < n_splits; ++sp) {          // in split order
-            const float wgt = __shfl(my_w, sp, 64);
-            l = fmaf(__shfl(my_l, sp, 64), wgt, l);
-            const float* pm = pp + ((size_t)sp * 2 + mp) * (DV + 2);
+        my_m[mp] = lane < n_splits ? mine[0] : -INFINITY;
+        my_l[mp] = lane < n_splits ? mine[1] : 0.f;
+    }
+    float my_w[2], l[2] = {0.f, 0.f}, a[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                if (lane + 64 * i < DV) a[i] = fmaf(pm[2 + lane + 64 * i], wgt, a[i]);
+    for (int mp = 0; mp < 2; ++mp) {
+        const float m = wave_max(my_m[mp]);
+        my_w[mp] = (my_m[mp] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((my_m[mp] - m) * scale2);
+    }
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {           // eight splits' rows of both maps asked for at once
+        float raw[8][2][4];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int mp = 0; mp < 2; ++mp) {
+                const float* pm = pp + ((size_t)min(s0 + j, n_splits - 1) * 2 + mp) * (DV + 2);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) raw[j][mp][i] = lane + 64 * i < DV ? pm[2 + lane + 64 * i] : 0.f;
+            }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {                    // in split order
+            if (s0 + j >= n_splits) break;
+#pragma unroll
+            for (int mp = 0; mp < 2; ++mp) {
+                const float wgt = __shfl(my_w[mp], s0 + j, 64);
+                l[mp] = fmaf(__shfl(my_l[mp], s0 + j, 64), wgt, l[mp]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[mp][i] = fmaf(raw[j][mp][i], wgt, a[mp][i]);
+            }
         }
-        const float f = l > 0.f ? (mp == 0 ? 1.0f : -lambda) / l : 0.f;
+    }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = fmaf(a[i], f, o[i]);
+    for (int mp = 0; mp < 2; ++mp) {
+        const float f = l[mp] > 0.f ? (mp == 0 ? 1.0f : -lambda) / l[mp] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = fmaf(a[mp][i], f, o[i]);
     }
     float ss = 0.f;
 #pragma unroll
@@ -427,7 +466,7 @@ __global__ __launch_bounds__(64) void attn_diff_merge_kernel(const float* __rest
         if (lane + 64 * i < DV) ss = fmaf(o[i], o[i], ss);
     ss = wave_sum(ss);
     const float f = out_scale / sqrtf(ss / (float)DV + eps);
-    bf16* op = out + ((size_t)cu_q[tiles[2 * tile]] * Hq + head) * DV;
+    bf16* op = out + ((size_t)token_row * Hq + head) * DV;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         if (lane + 64 * i < DV) op[lane + 64 * i] = from_f<bf16>(o[i] * f);
