@@ -17,7 +17,7 @@
 // qkv row: [Hq*M*D | Hkv*M*D | Hkv*Dv] (M maps). The first R elements of every map of q and k are rotated
 // by the token's position: interleaved (element 2i with 2i+1) or half-split (i with i + R/2); cos/sin are
 // [positions][R/2] in 32-bit. q goes to q_out [T][Hq*M*D], k to the key pool row of the token's slot, v to
-// the value pool row. One workgroup per token.
+// the value pool row. A workgroup per token and 1,024 elements of its row.
 template <typename T>
 __global__ void maps_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, int M, int D, int Dv,
                                     const int* __restrict__ positions, const float* __restrict__ cos_t,
@@ -30,7 +30,10 @@ __global__ void maps_prepare_kernel(const T* __restrict__ qkv, int Hq, int Hkv, 
     const int pos = positions[t];
     const int half = R >> 1;
     const long long slot = slot_mapping ? slot_mapping[t] : 0;
-    for (int c = threadIdx.x; c < qw + kw + vw; c += blockDim.x) {
+    // (a workgroup takes 1,024 elements of the token's row, a thread four of them: their reads are asked for together)
+    const int c_end = min(qw + kw + vw, ((int)blockIdx.y + 1) * 1024);
+#pragma unroll 4
+    for (int c = blockIdx.y * 1024 + threadIdx.x; c < c_end; c += 256) {
         if (c >= qw + kw) {                                   // a value
             if (v_pool == nullptr) continue;
             const int e = c - qw - kw, h = e / Dv;
@@ -65,7 +68,9 @@ extern "C" int ra_maps_qkv_prepare(const void* qkv, int T_tokens, int Hq, int Hk
     if (Hq <= 0 || Hkv <= 0 || M <= 0 || D <= 0 || Dv <= 0 || R < 0 || R > D || (R & 1) || P <= 0) return RA_ERR_ARG;
     if (R > 0 && (cos_t == nullptr || sin_t == nullptr)) return RA_ERR_ARG;
     if ((k_pool != nullptr || v_pool != nullptr) && slot_mapping == nullptr) return RA_ERR_ARG;
-    dim3 grid(T_tokens), block(256);
+    const long long len = (long long)(Hq + Hkv) * M * D + (long long)Hkv * Dv;
+    if (len > 65535LL * 1024) return RA_ERR_ARG;
+    dim3 grid(T_tokens, (unsigned)((len + 1023) / 1024)), block(256);
     if (dtype == RA_DTYPE_F32)
         hipLaunchKernelGGL(maps_prepare_kernel<float>, grid, block, 0, (hipStream_t)stream, (const float*)qkv, Hq, Hkv,
                            M, D, Dv, positions, cos_t, sin_t, R, interleaved, (float*)q_out, (float*)k_pool,
