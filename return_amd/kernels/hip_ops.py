@@ -1259,12 +1259,6 @@ class HipOps:
         tabs = (_ptr(g.page_table), _ptr(g.cu_pages), _ptr(g.kv_start), _ptr(step.cu_q), _ptr(step.q_start))
         consts = (float(scale), int(window), int(chunk), float(lam), float(eps), float(out_scale))
 
-        def plain(ids, ids_are_requests, rows):
-            self._check(self.lib.ra_attention_diff_plain(
-                _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(ids), 1 if ids_are_requests else 0,
-                step.n_seqs, rows, n_q, n_kv, D2 // 2, Dv, P, *consts, _code(q.dtype), self._stream()),
-                "attention_diff_plain")
-
         if q.dtype == torch.bfloat16 and scale > 0 and self.lib.ra_attention_diff_mfma_fits(D2 // 2, Dv):
             # the matrix-core kernel, tile by tile: the q tiles of the requests with two or more new tokens, and
             # one tile of one row for every request that brings a single token
@@ -1292,7 +1286,10 @@ class HipOps:
                     _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, _ptr(tiles), tiles.shape[0], n_q, n_kv,
                     D2 // 2, Dv, P, *consts, splits, _ptr(part), pack, self._stream()), "attention_diff_mfma_bf16")
             return
-        plain(None, False, T)
+        # float32, and sizes the matrix-core kernel does not take: the plain kernel over all rows of the step
+        self._check(self.lib.ra_attention_diff_plain(
+            _ptr(q), _ptr(out), _ptr(k_pool), _ptr(v_pool), *tabs, None, 0, step.n_seqs, T, n_q, n_kv, D2 // 2, Dv, P,
+            *consts, _code(q.dtype), self._stream()), "attention_diff_plain")
 
     def _diff_decode_splits(self, step, n_heads, window, chunk):
         """Workgroups that share the keys of a request that brings one token: enough of them to fill the chip
