@@ -58,7 +58,40 @@ RUPE_C_INIT = dict(seed=23, std=0.12, embedding_std=1.0, norm_jitter=0.05)
 CASES = {"a": (RUPE_A, RUPE_A_INIT), "b": (RUPE_B, RUPE_B_INIT), "c": (RUPE_C, RUPE_C_INIT)}
 
 
+def random_case(seed):
+    """A configuration drawn from a seed: one to four layers, every size and option drawn on its own (sizes that the
+    matrix-core kernels take and sizes they do not, value rows of any width beside the maps, chunks from 1 on, with
+    and without rotation, mask, feed-forward, groups, loop)."""
+    import random
+    rng = random.Random(seed)
+    n_layers = rng.choice([1, 2, 3, 4])
+    layers = []
+    for _ in range(n_layers):
+        kv = rng.choice([1, 1, 2, 3])
+        heads = kv * rng.choice([1, 2, 4, 5, 18] if kv == 1 else [1, 2, 4])
+        if rng.random() < 0.5:
+            dim, vdim = rng.choice([16, 32, 48, 64]), rng.choice([32, 64, 96, 128])
+        else:
+            dim, vdim = rng.choice([2, 4, 6, 10, 24, 40]), rng.choice([2, 5, 8, 20, 33, 48])
+        chunk = rng.choice([None, 1, 2, 5, 16, 31, 32, 64, 100, 128])
+        rot = (rng.choice([10.0, 10000.0, 1e6]), rng.choice(range(2, dim + 1, 2))) if rng.random() < 0.8 else None
+        moe = None
+        if rng.random() < 0.8:
+            count, per = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 3, 5])
+            keep = rng.randint(1, count)
+            moe = (rng.choice([4, 8, 12, 24, 40]), count * per, rng.randint(1, min(keep * per, 6)), count, keep)
+        layers.append(_layer(heads, kv, dim, vdim, rng.choice([dim ** -0.5, 0.3, 2.0 / dim]), rng.choice([0.1, 0.35, 0.5, 0.8]),
+                             chunk=chunk, rot=rot, moe=moe))
+    raw = {"architecture": "Rupezen", "vocab": rng.choice([50, 97, 256]), "width": rng.choice([16, 24, 40, 64, 96, 200]),
+           "norm": {"eps": rng.choice([1e-6, 1e-5])}, "residual_mult": rng.choice([0.5, 1.0, 0.7, 1.5]), "layers": layers}
+    if rng.random() < 0.7:
+        start = rng.randrange(0, n_layers)
+        raw["loop"] = {"start": start, "stop": rng.randint(start + 1, n_layers), "times": rng.choice([1, 2, 3])}
+    return raw, dict(seed=seed, std=0.15, embedding_std=1.0, norm_jitter=0.1)
+
+
 def make_folder(tmp_path_factory, name, dtype="bfloat16"):
     from tests.conftest import make_folder as make
-    raw, init = CASES[name]
+    raw, init = random_case(name) if isinstance(name, int) else CASES[name]
+    name = str(name)
     return make(tmp_path_factory, "rupezen_" + name, dict(raw, architectures=[raw["architecture"]]), init, dtype)
